@@ -63,6 +63,24 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
     return total;
 }
 
+// ---- gates of feed-forwards -------------------------------------------------------
+// What a gated feed-forward makes of its gate and up products g and u:
+//   TQK_GATE_SILU     g sigmoid(g) u
+//   TQK_GATE_RELU     max(g, 0) u
+//   TQK_GATE_CLAMPED  g' sigmoid(alpha g') (u' + 1) with g' = min(g, limit), u' = clamp(u, -limit, limit)
+//   TQK_GATE_GELU     gelu_tanh(g) u
+enum { TQK_GATE_SILU = 0, TQK_GATE_RELU = 1, TQK_GATE_CLAMPED = 2, TQK_GATE_GELU = 3, TQK_GATE_KINDS = 4 };
+__device__ __forceinline__ float gate_value(int kind, float limit, float alpha, float g, float u) {
+    if (kind == TQK_GATE_RELU) return fmaxf(g, 0.f) * u;
+    if (kind == TQK_GATE_CLAMPED) {
+        g = fminf(g, limit);
+        u = fminf(fmaxf(u, -limit), limit);
+        return (g / (1.f + expf(-alpha * g))) * (u + 1.f);
+    }
+    if (kind == TQK_GATE_GELU) return 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))) * u;
+    return (g / (1.f + expf(-g))) * u;
+}
+
 // ---- host side ------------------------------------------------------------------
 enum { TQK_F32 = 0, TQK_BF16 = 1 };
 

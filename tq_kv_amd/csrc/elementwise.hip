@@ -616,17 +616,18 @@ extern "C" int tqk_rope_store_sums(const float* sums, int n_sums, const void* bi
 // ---- SwiGLU ----------------------------------------------------------------------
 // silu(gate) * up, src/models/turbo_generic.rs:105-111 and :64-66.
 template <typename TA>
-__global__ void swiglu_kernel(const TA* __restrict__ gate_up, TA* __restrict__ out, int inter, size_t total) {
+__global__ void swiglu_kernel(const TA* __restrict__ gate_up, TA* __restrict__ out, int inter, size_t total, int kind, float limit, float alpha) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= total) return;
     const size_t t = i / inter, c = i % inter;
     const float g = to_float(gate_up[t * 2 * inter + c]);
     const float u = to_float(gate_up[t * 2 * inter + inter + c]);
-    out[i] = from_float<TA>((g / (1.f + expf(-g))) * u);
+    out[i] = from_float<TA>(gate_value(kind, limit, alpha, g, u));
 }
 
 // The same, 8 bfloat16 values (16 bytes) per thread; inter must be a multiple of 8.
-__global__ void swiglu_bf16x8_kernel(const uint4* __restrict__ gate_up, uint4* __restrict__ out, int inter8, size_t total8) {
+__global__ void swiglu_bf16x8_kernel(const uint4* __restrict__ gate_up, uint4* __restrict__ out, int inter8, size_t total8, int kind, float limit,
+                                     float alpha) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= total8) return;
     const size_t t = i / inter8, c = i % inter8;
@@ -637,26 +638,33 @@ __global__ void swiglu_bf16x8_kernel(const uint4* __restrict__ gate_up, uint4* _
     for (int k = 0; k < 4; ++k) {
         const float g0 = __uint_as_float(gw[k] << 16), g1 = __uint_as_float(gw[k] & 0xffff0000u);
         const float u0 = __uint_as_float(uw[k] << 16), u1 = __uint_as_float(uw[k] & 0xffff0000u);
-        const float r0 = (g0 / (1.f + expf(-g0))) * u0, r1 = (g1 / (1.f + expf(-g1))) * u1;
+        const float r0 = gate_value(kind, limit, alpha, g0, u0), r1 = gate_value(kind, limit, alpha, g1, u1);
         ow[k] = (uint32_t)float_to_bf16_bits(r0) | ((uint32_t)float_to_bf16_bits(r1) << 16);
     }
     out[i] = make_uint4(ow[0], ow[1], ow[2], ow[3]);
 }
 
 extern "C" int tqk_swiglu(const void* gate_up, void* out, int act_dtype, int n_tokens, int inter, void* stream) {
-    TQK_REQUIRE(gate_up && out, "tqk_swiglu: null pointer");
-    TQK_REQUIRE(n_tokens >= 0 && inter > 0, "tqk_swiglu: bad sizes");
+    return tqk_gated_act(gate_up, out, act_dtype, n_tokens, inter, TQK_GATE_SILU, 0.f, 1.f, stream);
+}
+
+extern "C" int tqk_gated_act(const void* gate_up, void* out, int act_dtype, int n_tokens, int inter, int kind, float limit, float alpha,
+                             void* stream) {
+    TQK_REQUIRE(gate_up && out, "tqk_gated_act: null pointer");
+    TQK_REQUIRE(n_tokens >= 0 && inter > 0, "tqk_gated_act: bad sizes");
+    TQK_REQUIRE(kind >= 0 && kind < TQK_GATE_KINDS, "tqk_gated_act: unknown gate %d", kind);
     if (n_tokens == 0) return 0;
     const size_t total = (size_t)n_tokens * inter;
     hipStream_t s = (hipStream_t)stream;
     if (act_dtype == TQK_BF16 && inter % 8 == 0 && ((((uintptr_t)gate_up) | ((uintptr_t)out)) & 15) == 0) {
         const size_t total8 = total / 8;
-        swiglu_bf16x8_kernel<<<(unsigned)((total8 + 255) / 256), 256, 0, s>>>((const uint4*)gate_up, (uint4*)out, inter / 8, total8);
-        return tqk_check_launch("tqk_swiglu");
+        swiglu_bf16x8_kernel<<<(unsigned)((total8 + 255) / 256), 256, 0, s>>>((const uint4*)gate_up, (uint4*)out, inter / 8, total8, kind, limit, alpha);
+        return tqk_check_launch("tqk_gated_act");
     }
     const unsigned blocks = (unsigned)((total + 255) / 256);
-    if (act_dtype == TQK_F32) swiglu_kernel<float><<<blocks, 256, 0, s>>>((const float*)gate_up, (float*)out, inter, total);
-    else if (act_dtype == TQK_BF16) swiglu_kernel<bf16_t><<<blocks, 256, 0, s>>>((const bf16_t*)gate_up, (bf16_t*)out, inter, total);
-    else return tqk_fail("tqk_swiglu: unknown dtype %d", act_dtype);
-    return tqk_check_launch("tqk_swiglu");
+    if (act_dtype == TQK_F32) swiglu_kernel<float><<<blocks, 256, 0, s>>>((const float*)gate_up, (float*)out, inter, total, kind, limit, alpha);
+    else if (act_dtype == TQK_BF16)
+        swiglu_kernel<bf16_t><<<blocks, 256, 0, s>>>((const bf16_t*)gate_up, (bf16_t*)out, inter, total, kind, limit, alpha);
+    else return tqk_fail("tqk_gated_act: unknown dtype %d", act_dtype);
+    return tqk_check_launch("tqk_gated_act");
 }

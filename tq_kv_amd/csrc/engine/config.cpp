@@ -15,7 +15,7 @@ std::vector<Architecture>& architectures() {
     return a;
 }
 std::once_flag g_builtin_once;
-void ensure_builtin() { std::call_once(g_builtin_once, [] { register_qwen2(); }); }
+void ensure_builtin() { std::call_once(g_builtin_once, [] { register_qwen2(); register_nikasun(); }); }
 std::string joined(const std::vector<std::string>& v) {
     std::string s;
     for (size_t i = 0; i < v.size(); ++i) s += (i ? ", " : "") + v[i];
@@ -43,6 +43,13 @@ const Architecture& architecture_for(const Json& raw) {
     const Json& archs = raw["architectures"];
     if (archs.is_array() && !archs.items().empty()) {
         const std::string name = archs.items()[0].is_string() ? archs.items()[0].as_string() : archs.items()[0].dump();
+        for (const Architecture& a : architectures())
+            if (a.name == name) return a;
+        raise(TQE_ERR_CONFIG, "Unknown architecture '%s'. Known architectures: %s", name.c_str(), joined(known_architectures()).c_str());
+    }
+    // some checkpoints name their one architecture in a string
+    if (raw["architecture"].is_string()) {
+        const std::string name = raw["architecture"].as_string();
         for (const Architecture& a : architectures())
             if (a.name == name) return a;
         raise(TQE_ERR_CONFIG, "Unknown architecture '%s'. Known architectures: %s", name.c_str(), joined(known_architectures()).c_str());

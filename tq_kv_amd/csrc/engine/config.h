@@ -28,5 +28,6 @@ std::vector<int32_t> generation_config_stop_ids(const std::string& model_dir);
 std::vector<int32_t> tokenizer_stop_ids(const std::string& model_dir);
 
 void register_qwen2();
+void register_nikasun();
 
 }  // namespace tq

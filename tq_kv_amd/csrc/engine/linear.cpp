@@ -112,11 +112,11 @@ static void k_fused_store(StepContext& c, const Tensor& x, const int32_t* rows, 
                    out.data, out.dtype, (int)out.shape[0], (int)w.n, (int)w.k, c.stream);
 }
 
-static void k_fused_gated(StepContext& c, const Tensor& x, const LazyNorm* norm, const Weight& w, Tensor& out) {
+static void k_fused_gated(StepContext& c, const Tensor& x, const LazyNorm* norm, const Weight& w, Tensor& out, const Gate& gate) {
     int packed = 0;
     const void* wp = few_ptr(w, &packed);
-    K::fused_gated(x.data, norm ? (const float*)norm->ss.data : nullptr, norm ? norm->n_ss : 0, norm ? norm->eps : 0.f, wp, packed, out.data,
-                   (int)out.shape[0], (int)w.n, (int)w.k, c.stream);
+    K::fused_gated_act(x.data, norm ? (const float*)norm->ss.data : nullptr, norm ? norm->n_ss : 0, norm ? norm->eps : 0.f, wp, packed, out.data,
+                       (int)out.shape[0], (int)w.n, (int)w.k, gate.kind, gate.limit, gate.alpha, c.stream);
 }
 
 // the product through the kernel for mid-sized steps; leave: its sums where it cuts K into pieces
@@ -138,12 +138,12 @@ static Product k_mid_store(StepContext& c, const Tensor& x, const Weight& w, int
     return p;
 }
 
-static void k_mid_gated(StepContext& c, const Tensor& x, const Weight& w, Tensor& out) {
+static void k_mid_gated(StepContext& c, const Tensor& x, const Weight& w, Tensor& out, const Gate& gate) {
     const int64_t m = x.shape[0];
     const int splits = K::mid_splits.raw((int)w.n, (int)w.k, 1);
     Tensor scratch;
     if (splits > 1) scratch = c.alloc(F32, {splits, m, w.n});
-    K::mid_gated(x.data, w.packed->t.data, out.data, (int)m, (int)w.n, (int)w.k, scratch.data, c.stream);
+    K::mid_gated_act(x.data, w.packed->t.data, out.data, (int)m, (int)w.n, (int)w.k, scratch.data, gate.kind, gate.limit, gate.alpha, c.stream);
 }
 
 static void k_gemm(StepContext& c, const Tensor& x, const Tensor& w, const Tensor* bias, Tensor& out) {
@@ -167,7 +167,7 @@ Product linear(StepContext& c, const Tensor& x, const Weight& w, const Tensor* b
             return p;
         }
         if (mid_ok(x, w)) return k_mid_store(c, x, w, out_dtype, leave_sums, out);
-        if (!w.rows && m > mid_max_rows() && policy().library && !null_device()) {
+        if (!w.rows && m > mid_max_rows() && policy().library && !null_device() && w.n % 8 == 0) {
             // the rows were given up and this is a prompt: the rows come back for the length of this product (the weight
             // read and written once more, against reading it once per 128 rows of x)
             Tensor rows = c.alloc(BF16, {w.n, w.k});
@@ -187,7 +187,8 @@ Product linear(StepContext& c, const Tensor& x, const Weight& w, const Tensor* b
             }
             return p;
         }
-        if (policy().library && m > skinny_max_rows() && !null_device()) {
+        // (rows of the operands and of the result at multiples of 16 bytes: what the library's kernels take for sure)
+        if (policy().library && m > skinny_max_rows() && !null_device() && w.k % 8 == 0 && w.n % 8 == 0) {
             p.t = out ? *out : c.alloc(out_dtype, {m, w.n});
             library_gemm(x, w.rows->t, p.t, c.stream);
             return p;
@@ -200,22 +201,65 @@ Product linear(StepContext& c, const Tensor& x, const Weight& w, const Tensor* b
     return p;
 }
 
-Tensor gated_silu_linear(StepContext& c, const Tensor& x, const Weight& w) {
+Gate Gate::from_params(const KeyReader& r, const char* what) {
+    Gate g;
+    const std::string name = r.string_or("gate", "silu");
+    if (name == "silu") g.kind = SiLU;
+    else if (name == "relu") g.kind = ReLU;
+    else if (name == "clamped") g.kind = Clamped;
+    else if (name == "gelu_tanh") g.kind = GELU;
+    else raise(TQE_ERR_ARGUMENT, "%s: unknown gate '%s' (known: silu, relu, clamped, gelu_tanh)", what, name.c_str());
+    if (g.kind == Clamped) {
+        g.limit = (float)r.number("limit", true);
+        g.alpha = (float)r.number_or("alpha", 1.0, true);
+    }
+    return g;
+}
+
+OwnedPtr stack_rows(const std::vector<OwnedPtr>& parts, hipStream_t stream, int64_t pad_rows_to) {
+    int dtype = parts[0]->t.dtype;
+    int64_t rows = 0;
+    for (const OwnedPtr& p : parts) {
+        if (p->t.dtype == F32) dtype = F32;
+        rows += p->t.shape[0];
+    }
+    const int64_t padded = (rows + pad_rows_to - 1) / pad_rows_to * pad_rows_to;
+    std::vector<int64_t> dims = {padded};
+    if (parts[0]->t.ndim == 2) dims.push_back(parts[0]->t.shape[1]);
+    OwnedPtr out = make_owned(dtype, dims);
+    int64_t at = 0;
+    for (const OwnedPtr& p : parts) {
+        Tensor dst = out->t.slice(at, at + p->t.shape[0]);
+        if (p->t.cols() != out->t.cols()) raise(TQE_ERR_WEIGHTS, "stacked tensors of different widths: %s under %s", p->t.describe().c_str(), parts[0]->t.describe().c_str());
+        if (p->t.dtype == dtype) copy_on_device(dst.data, p->t.data, p->t.bytes(), stream);
+        else if (null_device()) raise(TQE_ERR_WEIGHTS, "stacked tensors of different types cannot be converted without a GPU");
+        else K::convert(p->t.data, p->t.dtype, dst.data, dtype, (long long)p->t.numel(), stream);
+        at += p->t.shape[0];
+    }
+    if (padded > rows) {
+        Tensor rest = out->t.slice(rows, padded);
+        zero_device(rest.data, rest.bytes(), stream);
+    }
+    stream_synchronize(stream);
+    return out;
+}
+
+Tensor gated_linear(StepContext& c, const Tensor& x, const Weight& w, const Gate& gate) {
     const int64_t m = x.shape[0], inter = w.n / 2;
     Tensor act = c.alloc(x.dtype, {m, inter});
-    if (skinny_ok(x, w)) { k_fused_gated(c, x, nullptr, w, act); return act; }
-    if (mid_ok(x, w)) { k_mid_gated(c, x, w, act); return act; }
-    if (!w.rows && !(m > mid_max_rows() && policy().library && !null_device())) {
+    if (skinny_ok(x, w)) { k_fused_gated(c, x, nullptr, w, act, gate); return act; }
+    if (mid_ok(x, w)) { k_mid_gated(c, x, w, act, gate); return act; }
+    if (!w.rows && !(m > mid_max_rows() && policy().library && !null_device() && w.n % 8 == 0)) {
         const int64_t step = mid_max_rows();
         for (int64_t r = 0; r < m; r += step) {
             Tensor xs = x.slice(r, std::min(m, r + step)), os = act.slice(r, std::min(m, r + step));
-            if (xs.shape[0] <= skinny_max_rows()) k_fused_gated(c, xs, nullptr, w, os);
-            else k_mid_gated(c, xs, w, os);
+            if (xs.shape[0] <= skinny_max_rows()) k_fused_gated(c, xs, nullptr, w, os, gate);
+            else k_mid_gated(c, xs, w, os, gate);
         }
         return act;
     }
     Product both = linear(c, x, w, nullptr, x.dtype);
-    K::swiglu(both.t.data, act.data, act.dtype, (int)m, (int)inter, c.stream);
+    K::gated_act(both.t.data, act.data, act.dtype, (int)m, (int)inter, gate.kind, gate.limit, gate.alpha, c.stream);
     return act;
 }
 

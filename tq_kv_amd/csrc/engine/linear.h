@@ -64,8 +64,21 @@ struct Product {
 // x [M, K] times weight^T -> [M, N] of out_dtype (into `out` if given, else workspace memory).
 // leave_sums: the caller also takes the product unfinished where the kernel cuts K into pieces.
 Product linear(StepContext& c, const Tensor& x, const Weight& w, const Tensor* bias, int out_dtype, bool leave_sums = false, Tensor* out = nullptr);
-// silu(x Wg^T) * (x Wu^T) with Wg stacked on Wu: [M, K] x [2I, K] -> [M, I]
-Tensor gated_silu_linear(StepContext& c, const Tensor& x, const Weight& w_gate_up);
+// Which gate a gated feed-forward applies to its gate and up products g and u (the kernels' TQK_GATE_* codes):
+// silu g sigmoid(g) u; relu max(g, 0) u; clamped g' sigmoid(alpha g') (u' + 1) with g' = min(g, limit) and
+// u' = clamp(u, -limit, limit); gelu gelu_tanh(g) u.
+struct Gate {
+    enum Kind { SiLU = 0, ReLU = 1, Clamped = 2, GELU = 3 };
+    int kind = SiLU;
+    float limit = 0.f, alpha = 1.f;
+    static Gate from_params(const KeyReader& r, const char* what);      // "gate" (default "silu"), "limit", "alpha"
+};
+// gate(x Wg^T, x Wu^T) with Wg stacked on Wu: [M, K] x [2I, K] -> [M, I]
+Tensor gated_linear(StepContext& c, const Tensor& x, const Weight& w_gate_up, const Gate& gate);
+inline Tensor gated_silu_linear(StepContext& c, const Tensor& x, const Weight& w_gate_up) { return gated_linear(c, x, w_gate_up, Gate()); }
+// Several loaded tensors stacked along their first dimension (float32 if any of them is), then zero rows up to a
+// multiple of pad_rows_to.
+OwnedPtr stack_rows(const std::vector<OwnedPtr>& parts, hipStream_t stream, int64_t pad_rows_to = 1);
 // h += bfloat16(x weight^T), preparing stream.next_norm (small steps: in the product's epilogue;
 // mid-sized ones: left pending for the next norm's kernel, as sums where that norm takes them)
 void add_product(StepContext& c, Stream& stream, const Tensor& x, const Weight& w);

@@ -215,5 +215,7 @@ template <typename T> std::shared_ptr<T> build(const char* category, const PartS
     return p;
 }
 void register_builtin_parts();          // idempotent
+void register_latent_parts();           // parts_latent.cpp; called by register_builtin_parts
+void register_moe_parts();              // parts_moe.cpp; likewise
 
 }  // namespace tq

@@ -89,22 +89,49 @@ static OwnedPtr take(Loaded& tensors, const char* name) {
 // ---- RMSNorm -----------------------------------------------------------------------------------
 // As the reference computes it (src/models/turbo_generic.rs:41-51): x / sqrt(mean(x^2) + eps) *
 // weight in float32, cast last; the weight is used as it is stored (no 1 + w).
+//
+// params: size, eps; optional unit_offset (true: the stored weight lies around zero and the norm multiplies by
+// 1 + w; the sum is formed once, in float32, when the weight is loaded) and tensor (the name of the weight inside
+// the part's prefix, "weight" unless given; it may be empty where the prefix is the whole name).
 class RMSNorm : public Norm {
 public:
     RMSNorm(const PartSpec& spec, BuildEnv& env) : act_dtype_(env.act_dtype) {
         KeyReader r(spec.params, "rms_norm", TQE_ERR_ARGUMENT);
         size_ = r.integer("size", 1);
         eps_ = (float)r.number("eps");
+        unit_offset_ = r.boolean_or("unit_offset", false);
+        tensor_ = r.string_or("tensor", "weight");
         graph_safe = true;
     }
     TensorSpecs tensors() const override {
         TensorSpec t;
         t.shape = {size_};
-        t.init = "one_plus_normal";
-        return {{"weight", t}};
+        t.init = unit_offset_ ? "normal" : "one_plus_normal";
+        if (unit_offset_) t.std_dev = 0.1;
+        return {{tensor_, t}};
     }
-    void load(Loaded& tensors, hipStream_t) override { weight_ = take(tensors, "weight"); }
-    OwnedPtr held(const std::string& name) const override { return name == "weight" ? weight_ : nullptr; }
+    void load(Loaded& tensors, hipStream_t stream) override {
+        stored_ = take(tensors, tensor_.c_str());
+        weight_ = stored_;
+        if (!unit_offset_) return;
+        // 1 + w in float32, made on the host (a vector of the model's width, once)
+        const Tensor& t = stored_->t;
+        std::vector<float> host((size_t)t.numel());
+        if (t.dtype == F32) copy_to_host(host.data(), t.data, t.bytes(), stream);
+        else {
+            std::vector<uint16_t> bits((size_t)t.numel());
+            copy_to_host(bits.data(), t.data, t.bytes(), stream);
+            for (size_t i = 0; i < bits.size(); ++i) {
+                const uint32_t u = (uint32_t)bits[i] << 16;
+                memcpy(&host[i], &u, 4);
+            }
+        }
+        for (float& v : host) v = 1.0f + v;
+        weight_ = make_owned(F32, {size_});
+        copy_to_device(weight_->t.data, host.data(), host.size() * 4, stream);
+        stream_synchronize(stream);
+    }
+    OwnedPtr held(const std::string& name) const override { return name == tensor_ ? stored_ : name == "weight.effective" ? weight_ : nullptr; }
     const char* trace_name() const override { return "rms-norm"; }          // the reference's span, src/models/turbo_generic.rs:36
     int64_t size() const override { return size_; }
 
@@ -126,7 +153,9 @@ private:
     int64_t size_;
     float eps_;
     int act_dtype_;
-    OwnedPtr weight_;
+    bool unit_offset_;
+    std::string tensor_;
+    OwnedPtr stored_, weight_;       // what the checkpoint holds; what the kernels multiply by
 };
 
 // ---- positions ---------------------------------------------------------------------------------
@@ -251,28 +280,7 @@ public:
         return t;
     }
 
-    // several loaded tensors stacked along their first dimension: float32 if any of them is
-    static OwnedPtr stacked(const std::vector<OwnedPtr>& parts, hipStream_t stream) {
-        int dtype = parts[0]->t.dtype;
-        int64_t rows = 0;
-        for (const OwnedPtr& p : parts) {
-            if (p->t.dtype == F32) dtype = F32;
-            rows += p->t.shape[0];
-        }
-        std::vector<int64_t> dims = {rows};
-        if (parts[0]->t.ndim == 2) dims.push_back(parts[0]->t.shape[1]);
-        OwnedPtr out = make_owned(dtype, dims);
-        int64_t at = 0;
-        for (const OwnedPtr& p : parts) {
-            Tensor dst = out->t.slice(at, at + p->t.shape[0]);
-            if (p->t.dtype == dtype) copy_on_device(dst.data, p->t.data, p->t.bytes(), stream);
-            else if (null_device()) raise(TQE_ERR_WEIGHTS, "stacked tensors of different types cannot be converted without a GPU");
-            else K::convert(p->t.data, p->t.dtype, dst.data, dtype, (long long)p->t.numel(), stream);
-            at += p->t.shape[0];
-        }
-        stream_synchronize(stream);
-        return out;
-    }
+    static OwnedPtr stacked(const std::vector<OwnedPtr>& parts, hipStream_t stream) { return stack_rows(parts, stream); }
 
     void load(Loaded& t, hipStream_t stream) override {
         OwnedPtr qkv = stacked({take(t, "q_proj.weight"), take(t, "k_proj.weight"), take(t, "v_proj.weight")}, stream);
@@ -490,25 +498,34 @@ private:
     OwnedPtr b_qkv_, b_o_;
 };
 
-// ---- gated SiLU ----------------------------------------------------------------------------------
-// "SwiGLU" as the reference's Mlp (src/models/turbo_generic.rs:98-111): down(silu(gate(x)) * up(x)),
-// no biases.  Gate and up are one product with the weights stacked.  params: hidden, inter.
+// ---- gated feed-forward ----------------------------------------------------------------------------
+// down(gate(gate_proj(x), up_proj(x))), no biases.  With the SiLU gate this is "SwiGLU" as the reference's Mlp
+// (src/models/turbo_generic.rs:98-111): down(silu(gate(x)) * up(x)); kind "gated_silu" is that.  Kind "gated"
+// names its gate (params gate: silu, relu, clamped with limit and alpha, gelu_tanh; see Gate in linear.h).  Gate
+// and up are one product with the weights stacked.  params: hidden, inter; optional names {gate, up, down}: the
+// three tensors' names inside the part's prefix.
 class GatedSiLU : public FeedForward {
 public:
-    GatedSiLU(const PartSpec& spec, BuildEnv&) {
-        KeyReader r(spec.params, "gated_silu", TQE_ERR_ARGUMENT);
+    GatedSiLU(const PartSpec& spec, BuildEnv&, bool any_gate) {
+        KeyReader r(spec.params, any_gate ? "gated" : "gated_silu", TQE_ERR_ARGUMENT);
         hidden_ = r.integer("hidden", 1);
         inter_ = r.integer("inter", 1);
+        if (any_gate) gate_ = Gate::from_params(r, "gated");
+        const Json& names = spec.params["names"];
+        auto name = [&](const char* role, const char* fallback) { return names[role].is_string() ? names[role].as_string() : std::string(fallback); };
+        n_gate_ = name("gate", "gate_proj.weight");
+        n_up_ = name("up", "up_proj.weight");
+        n_down_ = name("down", "down_proj.weight");
         graph_safe = true;
     }
     TensorSpecs tensors() const override {
         auto w = [](int64_t a, int64_t b) { TensorSpec t; t.shape = {a, b}; return t; };
-        return {{"gate_proj.weight", w(inter_, hidden_)}, {"up_proj.weight", w(inter_, hidden_)}, {"down_proj.weight", w(hidden_, inter_)}};
+        return {{n_gate_, w(inter_, hidden_)}, {n_up_, w(inter_, hidden_)}, {n_down_, w(hidden_, inter_)}};
     }
     void load(Loaded& t, hipStream_t stream) override {
-        OwnedPtr gu = Attention::stacked({take(t, "gate_proj.weight"), take(t, "up_proj.weight")}, stream);
+        OwnedPtr gu = stack_rows({take(t, n_gate_.c_str()), take(t, n_up_.c_str())}, stream);
         w_gate_up_ = make_weight(gu, 2, false, stream);
-        w_down_ = make_weight(take(t, "down_proj.weight"), 1, false, stream);
+        w_down_ = make_weight(take(t, n_down_.c_str()), 1, false, stream);
     }
     OwnedPtr held(const std::string& name) const override {
         if (name == "gate_up.weight") return w_gate_up_.rows;
@@ -530,7 +547,7 @@ public:
 
     Tensor forward(StepContext& c, const Activation& x, Stream* stream) override {
         if (stream && !x.lazy && x.x.shape[0] > skinny_max_rows()) {
-            add_product(c, *stream, gated_silu_linear(c, x.x, w_gate_up_), w_down_);
+            add_product(c, *stream, gated_linear(c, x.x, w_gate_up_, gate_), w_down_);
             return Tensor();
         }
         if (x.lazy || stream) {
@@ -538,17 +555,19 @@ public:
             Tensor act = c.alloc(BF16, {xin.shape[0], inter_});
             int packed = 0;
             const void* wp = w_gate_up_.packed ? (packed = 1, w_gate_up_.packed->t.data) : w_gate_up_.rows->t.data;
-            K::fused_gated(xin.data, x.lazy ? (const float*)x.norm.ss.data : nullptr, x.lazy ? x.norm.n_ss : 0, x.lazy ? x.norm.eps : 0.f, wp, packed,
-                           act.data, (int)xin.shape[0], (int)(2 * inter_), (int)hidden_, c.stream);
+            K::fused_gated_act(xin.data, x.lazy ? (const float*)x.norm.ss.data : nullptr, x.lazy ? x.norm.n_ss : 0, x.lazy ? x.norm.eps : 0.f, wp,
+                               packed, act.data, (int)xin.shape[0], (int)(2 * inter_), (int)hidden_, gate_.kind, gate_.limit, gate_.alpha, c.stream);
             if (!stream) return linear(c, act, w_down_, nullptr, BF16).t;
             add_product(c, *stream, act, w_down_);
             return Tensor();
         }
-        return linear(c, gated_silu_linear(c, x.x, w_gate_up_), w_down_, nullptr, x.x.dtype).t;
+        return linear(c, gated_linear(c, x.x, w_gate_up_, gate_), w_down_, nullptr, x.x.dtype).t;
     }
 
 private:
     int64_t hidden_, inter_;
+    Gate gate_;
+    std::string n_gate_, n_up_, n_down_;
     Weight w_gate_up_, w_down_;
 };
 
@@ -582,12 +601,14 @@ public:
             return part;
         };
         mixer_ = std::dynamic_pointer_cast<Mixer>(one("mixer", "mixer", false));
-        feed_forward_ = std::dynamic_pointer_cast<FeedForward>(one("feed_forward", "feed_forward", false));
+        // a layer may have no feed-forward (feed_forward: null): then it has no norm in front of one either
+        const bool has_ff = !spec.params["feed_forward"].is_null();
+        feed_forward_ = std::dynamic_pointer_cast<FeedForward>(one("feed_forward", "feed_forward", true));
         mixer_norm_ = std::dynamic_pointer_cast<Norm>(one("mixer_norm", "norm", false));
-        ff_norm_ = std::dynamic_pointer_cast<Norm>(one("ff_norm", "norm", false));
+        ff_norm_ = has_ff ? std::dynamic_pointer_cast<Norm>(one("ff_norm", "norm", false)) : nullptr;
         post_mixer_norm_ = std::dynamic_pointer_cast<Norm>(one("post_mixer_norm", "norm", true));
-        post_ff_norm_ = std::dynamic_pointer_cast<Norm>(one("post_ff_norm", "norm", true));
-        if (!mixer_ || !feed_forward_ || !mixer_norm_ || !ff_norm_) raise(TQE_ERR_ARGUMENT, "pre_norm block: a part is of the wrong category");
+        post_ff_norm_ = has_ff ? std::dynamic_pointer_cast<Norm>(one("post_ff_norm", "norm", true)) : nullptr;
+        if (!mixer_ || (has_ff && (!feed_forward_ || !ff_norm_)) || !mixer_norm_) raise(TQE_ERR_ARGUMENT, "pre_norm block: a part is of the wrong category");
         graph_safe = true;
         for (const Role& r : roles_) graph_safe = graph_safe && r.part->graph_safe;
     }
@@ -630,9 +651,10 @@ public:
         {
             Span span(mixer_->trace_name());
             const bool adds = (c.fuse_small || c.fuse_mid) && !post_mixer_norm_ && mixer_->adds_to_stream(c);
-            if (adds) stream->next_norm = ff_norm_.get();
+            if (adds) stream->next_norm = feed_forward_ ? ff_norm_.get() : next_norm;
             settle(c, *stream, mixer_->forward(c, x, entry, adds ? stream : nullptr, false), post_mixer_norm_.get());
         }
+        if (!feed_forward_) return stream;
         x = normed(c, *ff_norm_, *stream, feed_forward_->folds_norm(c));
         {
             Span span(feed_forward_->trace_name());
@@ -691,6 +713,7 @@ private:
         if (c.n_last == 0) return sub;
         k_gather_rows(c, stream->h, c.dev.last_rows, c.n_last, sub->h);
         settle(c, *sub, y, post_mixer_norm_.get());
+        if (!feed_forward_) return sub;
         {
             Span span(ff_norm_->trace_name());
             x.x = c.alloc(c.act_dtype, {c.n_last, stream->h.shape[1]});
@@ -719,7 +742,10 @@ void register_builtin_parts() {
         register_kind("position", "rotary", [](const PartSpec& s, BuildEnv& e) { return std::make_shared<Rotary>(s, e); });
         register_kind("position", "none", [](const PartSpec& s, BuildEnv& e) { return std::make_shared<NoPosition>(s, e); });
         register_kind("mixer", "attention", [](const PartSpec& s, BuildEnv& e) { return std::make_shared<Attention>(s, e); });
-        register_kind("feed_forward", "gated_silu", [](const PartSpec& s, BuildEnv& e) { return std::make_shared<GatedSiLU>(s, e); });
+        register_kind("feed_forward", "gated_silu", [](const PartSpec& s, BuildEnv& e) { return std::make_shared<GatedSiLU>(s, e, false); });
+        register_kind("feed_forward", "gated", [](const PartSpec& s, BuildEnv& e) { return std::make_shared<GatedSiLU>(s, e, true); });
+        register_latent_parts();
+        register_moe_parts();
         register_kind("block", "pre_norm", [](const PartSpec& s, BuildEnv& e) { return std::make_shared<PreNormBlock>(s, e); });
     });
 }

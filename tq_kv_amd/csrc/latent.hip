@@ -1,0 +1,327 @@
+// Attention through a low-rank latent: the kernels around the cache of latents.
+//
+// Every position leaves one row in the cache, shared by all heads: the normed latent c [rk] and
+// one rotated key part r [dr].  A head's key would be (W_uk,h c, r) and its value W_uv,h c; neither
+// is ever formed.  Since q_h . (W_uk,h c) = (W_uk,h^T q_h) . c, the query is taken into the latent's
+// space once per token ("absorbed"), attention runs with the cache row as the key and its first rk
+// elements as the value, the same for every head, and W_uv,h is applied to the attended latent:
+//
+//   split      one row of the stacked first products [q latent | kv latent, rotated part | gate logits]:
+//              RMS norm of the q latent -> cq; RMS norm of the kv latent and rotation of the rotated part
+//              -> the cache row of the token's position; sigmoid of the gate logits -> gate [T, H]
+//   absorb     q [T, H, dn + dr] -> qa [T, H, rk + dr]: qa[:rk] = W_uk,h^T q[:dn], qa[rk:] = rotated q[dn:]
+//   attention  softmax((qa . row) * scale) over the window, times row[:rk] -> o [T, H, rk]
+//   values     y[t, h, :] = gate[t, h] * W_uv,h o[t, h, :]
+//
+// Norms, angles, scores, softmax weights, gates and all sums are float32; qa and o stay float32
+// between the kernels.  The order of a query's operations depends on its position alone.
+// Cache pages: [position in page][rk + dr].
+#include "common.h"
+#include "tq_kernels.h"
+
+#define LAT_MAX_RK 512          // largest latent the attention kernel's accumulators hold
+#define LAT_MAX_DK 640          // largest cache row (latent + rotated part)
+#define LAT_TT 8                // tokens a block of the absorb and values kernels takes
+
+// ---- split -----------------------------------------------------------------------------------
+template <typename TA, typename TW>
+__global__ __launch_bounds__(256)
+void latent_split_kernel(const TA* __restrict__ proj, int row_stride, int q_rank, int kv_rank, int rot_dim, int n_gate,
+                         const TW* __restrict__ q_norm_w, const TW* __restrict__ kv_norm_w, float eps,
+                         const float* __restrict__ cos_table, const float* __restrict__ sin_table, int rot_dims, int max_positions,
+                         const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos,
+                         const int32_t* __restrict__ page_table, int table_width, TA* __restrict__ cache, int n_pages,
+                         TA* __restrict__ cq_out, float* __restrict__ gate_out) {
+    __shared__ float scratch[8];
+    const int t = blockIdx.x;
+    const int kv_cols = kv_rank > 0 ? kv_rank + rot_dim : 0;
+    const TA* row = proj + (size_t)t * row_stride;
+    // the query's latent
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < q_rank; i += blockDim.x) { const float v = to_float(row[i]); ss = fmaf(v, v, ss); }
+    ss = block_sum(ss, scratch);
+    const float inv_q = 1.f / sqrtf(ss / (float)q_rank + eps);
+    for (int i = threadIdx.x; i < q_rank; i += blockDim.x)
+        cq_out[(size_t)t * q_rank + i] = from_float<TA>(to_float(row[i]) * inv_q * to_float(q_norm_w[i]));
+    // the gates
+    for (int i = threadIdx.x; i < n_gate; i += blockDim.x)
+        gate_out[(size_t)t * n_gate + i] = 1.f / (1.f + expf(-to_float(row[q_rank + kv_cols + i])));
+    if (kv_rank <= 0) return;
+    // the cache row
+    const TA* kv = row + q_rank;
+    ss = 0.f;
+    for (int i = threadIdx.x; i < kv_rank; i += blockDim.x) { const float v = to_float(kv[i]); ss = fmaf(v, v, ss); }
+    ss = block_sum(ss, scratch);
+    const float inv_kv = 1.f / sqrtf(ss / (float)kv_rank + eps);
+    const int pos = tok_pos[t];
+    const int page = page_table[(size_t)tok_seq[t] * table_width + pos / TQK_PAGE];
+    if (page < 0 || page >= n_pages) return;
+    TA* dst = cache + ((size_t)page * TQK_PAGE + (size_t)(pos % TQK_PAGE)) * kv_cols;
+    for (int i = threadIdx.x; i < kv_rank; i += blockDim.x) dst[i] = from_float<TA>(to_float(kv[i]) * inv_kv * to_float(kv_norm_w[i]));
+    const int half = rot_dims / 2;
+    const int p = min(pos, max_positions - 1);
+    for (int i = threadIdx.x; i < rot_dim; i += blockDim.x) {
+        const float v = to_float(kv[kv_rank + i]);
+        float r = v;
+        if (i < rot_dims) {
+            const int j = i < half ? i : i - half;
+            const float c = cos_table[(size_t)p * half + j], s = sin_table[(size_t)p * half + j];
+            const float other = to_float(kv[kv_rank + (i < half ? i + half : i - half)]);
+            r = i < half ? v * c - other * s : v * c + other * s;
+        }
+        dst[kv_rank + i] = from_float<TA>(r);
+    }
+}
+
+// ---- absorb ----------------------------------------------------------------------------------
+// A block: LAT_TT tokens of one head.  Thread j takes latent columns j, j + 128, ...; the head's rows
+// of W_uk are read along their columns, so a wave's loads are contiguous.
+template <typename TA, typename TW>
+__global__ __launch_bounds__(128)
+void latent_absorb_kernel(const TA* __restrict__ q, const TW* __restrict__ w_uk, int n_heads, int dn, int dr, int rk,
+                          const float* __restrict__ cos_table, const float* __restrict__ sin_table, int rot_dims, int max_positions,
+                          const int32_t* __restrict__ tok_pos, float* __restrict__ qa, int n_tokens) {
+    extern __shared__ float q_lds[];            // [LAT_TT][dn + dr]
+    const int head = blockIdx.y, t0 = blockIdx.x * LAT_TT, d = dn + dr;
+    const int n_t = min(LAT_TT, n_tokens - t0);
+    for (int i = threadIdx.x; i < LAT_TT * d; i += blockDim.x) {
+        const int tt = i / d, c = i % d;
+        q_lds[i] = tt < n_t ? to_float(q[((size_t)(t0 + tt) * n_heads + head) * d + c]) : 0.f;
+    }
+    __syncthreads();
+    const TW* w = w_uk + (size_t)head * dn * rk;
+    for (int j = threadIdx.x; j < rk; j += blockDim.x) {
+        float acc[LAT_TT];
+#pragma unroll
+        for (int tt = 0; tt < LAT_TT; ++tt) acc[tt] = 0.f;
+        for (int c = 0; c < dn; ++c) {
+            const float wv = to_float(w[(size_t)c * rk + j]);
+#pragma unroll
+            for (int tt = 0; tt < LAT_TT; ++tt) acc[tt] = fmaf(q_lds[tt * d + c], wv, acc[tt]);
+        }
+#pragma unroll
+        for (int tt = 0; tt < LAT_TT; ++tt)
+            if (tt < n_t) qa[((size_t)(t0 + tt) * n_heads + head) * (rk + dr) + j] = acc[tt];
+    }
+    const int half = rot_dims / 2;
+    for (int i = threadIdx.x; i < n_t * dr; i += blockDim.x) {
+        const int tt = i / dr, c = i % dr;
+        const float* qr = q_lds + tt * d + dn;
+        float r = qr[c];
+        if (c < rot_dims) {
+            const int p = min(tok_pos[t0 + tt], max_positions - 1);
+            const int j = c < half ? c : c - half;
+            const float cs = cos_table[(size_t)p * half + j], sn = sin_table[(size_t)p * half + j];
+            r = c < half ? qr[c] * cs - qr[c + half] * sn : qr[c] * cs + qr[c - half] * sn;
+        }
+        qa[((size_t)(t0 + tt) * n_heads + head) * (rk + dr) + rk + c] = r;
+    }
+}
+
+// ---- attention -------------------------------------------------------------------------------
+// One wave per (token, head).  Keys are taken a page at a time: lane j computes the score of the
+// page's position j, the softmax runs online over pages, then lane c accumulates element c
+// (+64, +128, ...) of the attended latent over the page's positions.
+#define LAT_WAVES 4
+template <typename TA>
+__global__ __launch_bounds__(LAT_WAVES * TQK_WAVE)
+void latent_attention_kernel(const float* __restrict__ qa, const TA* __restrict__ cache, const int32_t* __restrict__ tok_seq,
+                             const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ page_table, int table_width,
+                             int window, float scale, float* __restrict__ out, int n_tokens, int n_heads, int rk, int dk) {
+    __shared__ float q_lds[LAT_WAVES][LAT_MAX_DK];
+    const int wave = threadIdx.x / TQK_WAVE, lane = threadIdx.x % TQK_WAVE;
+    const int t = blockIdx.x * LAT_WAVES + wave;
+    const int head = blockIdx.y;
+    const bool live = t < n_tokens;
+    if (live) {
+        const float* qv = qa + ((size_t)t * n_heads + head) * dk;
+        for (int i = lane; i < dk; i += TQK_WAVE) q_lds[wave][i] = qv[i];
+    }
+    __syncthreads();
+    if (!live) return;
+    const int pos = tok_pos[t];
+    const int32_t* pages = page_table + (size_t)tok_seq[t] * table_width;
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const float* qf = q_lds[wave];
+    constexpr int NACC = LAT_MAX_RK / TQK_WAVE;
+    float acc[NACC];
+#pragma unroll
+    for (int i = 0; i < NACC; ++i) acc[i] = 0.f;
+    float m = -INFINITY, l = 0.f;
+    for (int kb = (lo / TQK_PAGE) * TQK_PAGE; kb <= pos; kb += TQK_PAGE) {
+        const int page = pages[kb / TQK_PAGE];
+        const int j = kb + lane;
+        const bool valid = j >= lo && j <= pos && page >= 0;
+        const TA* base = cache + (size_t)(page < 0 ? 0 : page) * TQK_PAGE * dk;
+        float s = -INFINITY;
+        if (valid) {
+            const TA* kr = base + (size_t)lane * dk;
+            float dot = 0.f;
+            for (int i = 0; i < dk; ++i) dot = fmaf(qf[i], to_float(kr[i]), dot);
+            s = dot * scale;
+        }
+        const float m_new = fmaxf(m, wave_max(s));
+        const float p = valid ? expf(s - m_new) : 0.f;
+        const float alpha = expf(m - m_new);
+        l = l * alpha + wave_sum(p);
+        m = m_new;
+        const int n_keys = min(TQK_PAGE, pos - kb + 1);
+        const int first_key = max(0, lo - kb);
+#pragma unroll
+        for (int a = 0; a < NACC; ++a) {
+            const int c = lane + a * TQK_WAVE;
+            float sum = acc[a] * alpha;
+            if (a * TQK_WAVE < rk) {
+                for (int jj = first_key; jj < n_keys; ++jj) {
+                    const float pj = __shfl(p, jj, TQK_WAVE);
+                    if (c < rk) sum = fmaf(pj, to_float(base[(size_t)jj * dk + c]), sum);
+                }
+            }
+            acc[a] = sum;
+        }
+    }
+    float* o = out + ((size_t)t * n_heads + head) * rk;
+#pragma unroll
+    for (int a = 0; a < NACC; ++a) {
+        const int c = lane + a * TQK_WAVE;
+        if (c < rk) o[c] = acc[a] / l;
+    }
+}
+
+// ---- values ----------------------------------------------------------------------------------
+// A block: LAT_TT tokens of one head; a wave takes value columns in turn, its lanes share a row of
+// W_uv (contiguous loads) and their partial sums are added up in a fixed order.
+template <typename TA, typename TW>
+__global__ __launch_bounds__(256)
+void latent_values_kernel(const float* __restrict__ o, const TW* __restrict__ w_uv, const float* __restrict__ gate, int n_heads, int rk,
+                          int dv, TA* __restrict__ y, int n_tokens) {
+    extern __shared__ float o_lds[];            // [LAT_TT][rk]
+    const int head = blockIdx.y, t0 = blockIdx.x * LAT_TT;
+    const int n_t = min(LAT_TT, n_tokens - t0);
+    for (int i = threadIdx.x; i < LAT_TT * rk; i += blockDim.x) {
+        const int tt = i / rk, c = i % rk;
+        o_lds[i] = tt < n_t ? o[((size_t)(t0 + tt) * n_heads + head) * rk + c] : 0.f;
+    }
+    __syncthreads();
+    const int wave = threadIdx.x / TQK_WAVE, lane = threadIdx.x % TQK_WAVE, n_waves = blockDim.x / TQK_WAVE;
+    for (int n = wave; n < dv; n += n_waves) {
+        const TW* w = w_uv + ((size_t)head * dv + n) * rk;
+        float acc[LAT_TT];
+#pragma unroll
+        for (int tt = 0; tt < LAT_TT; ++tt) acc[tt] = 0.f;
+        for (int c = lane; c < rk; c += TQK_WAVE) {
+            const float wv = to_float(w[c]);
+#pragma unroll
+            for (int tt = 0; tt < LAT_TT; ++tt) acc[tt] = fmaf(o_lds[tt * rk + c], wv, acc[tt]);
+        }
+#pragma unroll
+        for (int tt = 0; tt < LAT_TT; ++tt) acc[tt] = wave_sum(acc[tt]);
+        if (lane < n_t) {
+            float v = 0.f;
+#pragma unroll
+            for (int tt = 0; tt < LAT_TT; ++tt) v = lane == tt ? acc[tt] : v;
+            const int t = t0 + lane;
+            const float g = gate ? gate[(size_t)t * n_heads + head] : 1.f;
+            y[((size_t)t * n_heads + head) * dv + n] = from_float<TA>(v * g);
+        }
+    }
+}
+
+// ---- entry points ----------------------------------------------------------------------------
+extern "C" int tqk_latent_max_rank(void) { return LAT_MAX_RK; }
+extern "C" int tqk_latent_max_row(void) { return LAT_MAX_DK; }
+
+extern "C" int tqk_latent_split(const void* proj, int act_dtype, int row_stride, int q_rank, int kv_rank, int rot_dim, int n_gate, const void* q_norm_w,
+                                const void* kv_norm_w, int norm_dtype, float eps, const float* cos_table, const float* sin_table,
+                                int rot_dims, int max_positions, const int32_t* tok_seq, const int32_t* tok_pos,
+                                const int32_t* page_table, int table_width, void* cache, int n_pages, void* cq_out, float* gate_out,
+                                int n_tokens, void* stream) {
+    TQK_REQUIRE(proj && q_norm_w && cq_out, "tqk_latent_split: null pointer");
+    TQK_REQUIRE(q_rank > 0 && kv_rank >= 0 && rot_dim >= 0 && n_gate >= 0 && n_tokens >= 0, "tqk_latent_split: bad sizes");
+    TQK_REQUIRE(n_gate == 0 || gate_out, "tqk_latent_split: no place for the gates");
+    TQK_REQUIRE(row_stride >= q_rank + (kv_rank > 0 ? kv_rank + rot_dim : 0) + n_gate, "tqk_latent_split: rows of %d values are too short", row_stride);
+    if (kv_rank > 0) {
+        TQK_REQUIRE(kv_norm_w && cache && tok_seq && tok_pos && page_table && table_width > 0 && n_pages > 0, "tqk_latent_split: no cache to write");
+        TQK_REQUIRE(rot_dims >= 0 && rot_dims <= rot_dim && rot_dims % 2 == 0, "tqk_latent_split: %d of %d elements rotate", rot_dims, rot_dim);
+        TQK_REQUIRE(rot_dims == 0 || (cos_table && sin_table && max_positions > 0), "tqk_latent_split: no angle tables");
+    }
+    if (n_tokens == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+#define TQK_SPLIT(TA, TW)                                                                                                              \
+    latent_split_kernel<TA, TW><<<n_tokens, 256, 0, s>>>((const TA*)proj, row_stride, q_rank, kv_rank, rot_dim, n_gate, (const TW*)q_norm_w,       \
+                                                         (const TW*)kv_norm_w, eps, cos_table, sin_table, rot_dims, max_positions,     \
+                                                         tok_seq, tok_pos, page_table, table_width, (TA*)cache, n_pages, (TA*)cq_out,  \
+                                                         gate_out)
+    if (act_dtype == TQK_F32 && norm_dtype == TQK_F32) TQK_SPLIT(float, float);
+    else if (act_dtype == TQK_F32 && norm_dtype == TQK_BF16) TQK_SPLIT(float, bf16_t);
+    else if (act_dtype == TQK_BF16 && norm_dtype == TQK_F32) TQK_SPLIT(bf16_t, float);
+    else if (act_dtype == TQK_BF16 && norm_dtype == TQK_BF16) TQK_SPLIT(bf16_t, bf16_t);
+    else return tqk_fail("tqk_latent_split: unknown dtypes %d, %d", act_dtype, norm_dtype);
+#undef TQK_SPLIT
+    return tqk_check_launch("tqk_latent_split");
+}
+
+extern "C" int tqk_latent_absorb(const void* q, int act_dtype, const void* w_uk, int w_dtype, int n_heads, int dn, int dr, int rk,
+                                 const float* cos_table, const float* sin_table, int rot_dims, int max_positions,
+                                 const int32_t* tok_pos, float* qa, int n_tokens, void* stream) {
+    TQK_REQUIRE(q && w_uk && qa && tok_pos, "tqk_latent_absorb: null pointer");
+    TQK_REQUIRE(n_heads > 0 && n_heads <= 65535 && dn > 0 && dr >= 0 && rk > 0 && n_tokens >= 0, "tqk_latent_absorb: bad sizes");
+    TQK_REQUIRE(rot_dims >= 0 && rot_dims <= dr && rot_dims % 2 == 0, "tqk_latent_absorb: %d of %d elements rotate", rot_dims, dr);
+    TQK_REQUIRE(rot_dims == 0 || (cos_table && sin_table && max_positions > 0), "tqk_latent_absorb: no angle tables");
+    const size_t lds = (size_t)LAT_TT * (dn + dr) * sizeof(float);
+    TQK_REQUIRE(lds <= 48 * 1024, "tqk_latent_absorb: a head of %d + %d elements is more than the kernel stages", dn, dr);
+    if (n_tokens == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    dim3 grid((n_tokens + LAT_TT - 1) / LAT_TT, n_heads);
+#define TQK_ABSORB(TA, TW)                                                                                                             \
+    latent_absorb_kernel<TA, TW><<<grid, 128, lds, s>>>((const TA*)q, (const TW*)w_uk, n_heads, dn, dr, rk, cos_table, sin_table,      \
+                                                        rot_dims, max_positions, tok_pos, qa, n_tokens)
+    if (act_dtype == TQK_F32 && w_dtype == TQK_F32) TQK_ABSORB(float, float);
+    else if (act_dtype == TQK_F32 && w_dtype == TQK_BF16) TQK_ABSORB(float, bf16_t);
+    else if (act_dtype == TQK_BF16 && w_dtype == TQK_F32) TQK_ABSORB(bf16_t, float);
+    else if (act_dtype == TQK_BF16 && w_dtype == TQK_BF16) TQK_ABSORB(bf16_t, bf16_t);
+    else return tqk_fail("tqk_latent_absorb: unknown dtypes %d, %d", act_dtype, w_dtype);
+#undef TQK_ABSORB
+    return tqk_check_launch("tqk_latent_absorb");
+}
+
+extern "C" int tqk_latent_attention(const float* qa, const void* cache, int cache_dtype, const int32_t* tok_seq, const int32_t* tok_pos,
+                                    const int32_t* page_table, int table_width, int n_seqs, int n_pages, int window, float scale,
+                                    float* out, int n_tokens, int n_heads, int rk, int dr, void* stream) {
+    TQK_REQUIRE(qa && cache && tok_seq && tok_pos && page_table && out, "tqk_latent_attention: null pointer");
+    TQK_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_heads <= 65535 && rk > 0 && dr >= 0, "tqk_latent_attention: bad sizes");
+    TQK_REQUIRE(rk <= LAT_MAX_RK && rk + dr <= LAT_MAX_DK, "tqk_latent_attention: a latent of %d + %d is more than %d + %d", rk, dr, LAT_MAX_RK,
+                LAT_MAX_DK - LAT_MAX_RK);
+    TQK_REQUIRE(table_width > 0 && n_pages > 0 && n_seqs > 0 && window >= 0, "tqk_latent_attention: empty page table or negative window");
+    if (n_tokens == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    dim3 grid((n_tokens + LAT_WAVES - 1) / LAT_WAVES, n_heads);
+    if (cache_dtype == TQK_F32)
+        latent_attention_kernel<float><<<grid, LAT_WAVES * TQK_WAVE, 0, s>>>(qa, (const float*)cache, tok_seq, tok_pos, page_table, table_width,
+                                                                             window, scale, out, n_tokens, n_heads, rk, rk + dr);
+    else if (cache_dtype == TQK_BF16)
+        latent_attention_kernel<bf16_t><<<grid, LAT_WAVES * TQK_WAVE, 0, s>>>(qa, (const bf16_t*)cache, tok_seq, tok_pos, page_table, table_width,
+                                                                              window, scale, out, n_tokens, n_heads, rk, rk + dr);
+    else return tqk_fail("tqk_latent_attention: unknown dtype %d", cache_dtype);
+    return tqk_check_launch("tqk_latent_attention");
+}
+
+extern "C" int tqk_latent_values(const float* o, const void* w_uv, int w_dtype, const float* gate, int n_heads, int rk, int dv, void* y,
+                                 int y_dtype, int n_tokens, void* stream) {
+    TQK_REQUIRE(o && w_uv && y, "tqk_latent_values: null pointer");
+    TQK_REQUIRE(n_heads > 0 && n_heads <= 65535 && rk > 0 && dv > 0 && n_tokens >= 0, "tqk_latent_values: bad sizes");
+    const size_t lds = (size_t)LAT_TT * rk * sizeof(float);
+    TQK_REQUIRE(lds <= 48 * 1024, "tqk_latent_values: a latent of %d elements is more than the kernel stages", rk);
+    if (n_tokens == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    dim3 grid((n_tokens + LAT_TT - 1) / LAT_TT, n_heads);
+#define TQK_VALUES(TA, TW) \
+    latent_values_kernel<TA, TW><<<grid, 256, lds, s>>>(o, (const TW*)w_uv, gate, n_heads, rk, dv, (TA*)y, n_tokens)
+    if (y_dtype == TQK_F32 && w_dtype == TQK_F32) TQK_VALUES(float, float);
+    else if (y_dtype == TQK_F32 && w_dtype == TQK_BF16) TQK_VALUES(float, bf16_t);
+    else if (y_dtype == TQK_BF16 && w_dtype == TQK_F32) TQK_VALUES(bf16_t, float);
+    else if (y_dtype == TQK_BF16 && w_dtype == TQK_BF16) TQK_VALUES(bf16_t, bf16_t);
+    else return tqk_fail("tqk_latent_values: unknown dtypes %d, %d", y_dtype, w_dtype);
+#undef TQK_VALUES
+    return tqk_check_launch("tqk_latent_values");
+}

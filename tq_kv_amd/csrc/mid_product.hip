@@ -46,6 +46,8 @@ struct MidArgs {
     void* y;                    // store: [M, N]; gated: [M, N/2] bfloat16
     float* partial;             // [splits][M][N] when the grid has splits
     int M, N, K, k_per_split;   // k_per_split: a multiple of MID_CHUNK
+    int gate;                   // gated: which gate (TQK_GATE_*), with its limit and alpha
+    float gate_limit, gate_alpha;
 };
 
 __device__ __forceinline__ uint2 pack4_bf16(float a, float b, float c, float d) {
@@ -53,9 +55,10 @@ __device__ __forceinline__ uint2 pack4_bf16(float a, float b, float c, float d) 
                       (uint32_t)float_to_bf16_bits(c) | ((uint32_t)float_to_bf16_bits(d) << 16));
 }
 
-__device__ __forceinline__ float gate_times_up(float gate_sum, float up_sum) {
+struct Gate { int kind; float limit, alpha; };
+__device__ __forceinline__ float gate_times_up(const Gate& gate, float gate_sum, float up_sum) {
     const float g = to_float(from_float<bf16_t>(gate_sum)), up = to_float(from_float<bf16_t>(up_sum));
-    return (g / (1.f + expf(-g))) * up;
+    return gate_value(gate.kind, gate.limit, gate.alpha, g, up);
 }
 
 // MT: groups of 16 rows of x (2: up to 32 rows, 4: up to 64, 8: up to 128).  TN: tiles of 16
@@ -286,7 +289,7 @@ void mid_product_kernel(const MidArgs p) {
             if (m >= p.M) continue;
             float o[4];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) o[r] = gate_times_up(acc[0][mt][r], acc[TN - 1][mt][r]);
+            for (int r = 0; r < 4; ++r) o[r] = gate_times_up(Gate{p.gate, p.gate_limit, p.gate_alpha}, acc[0][mt][r], acc[TN - 1][mt][r]);
             bf16_t* dst = y + (size_t)m * n_out + n;
             if (vec && n + 3 < n_out) { *reinterpret_cast<uint2*>(dst) = pack4_bf16(o[0], o[1], o[2], o[3]); continue; }
 #pragma unroll
@@ -298,7 +301,7 @@ void mid_product_kernel(const MidArgs p) {
 
 // Adds the splits' sums in split order and finishes as the product kernel does without splits.
 template <int EPI, typename TY>
-__global__ void mid_finish_kernel(const float* __restrict__ partial, void* __restrict__ yv, int splits, int M, int N) {
+__global__ void mid_finish_kernel(const float* __restrict__ partial, void* __restrict__ yv, int splits, int M, int N, Gate gate) {
     const int n_out = EPI == MID_GATED ? N / 2 : N;
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= (size_t)M * n_out) return;
@@ -309,7 +312,7 @@ __global__ void mid_finish_kernel(const float* __restrict__ partial, void* __res
         a += src[n];
         if (EPI == MID_GATED) b += src[n_out + n];
     }
-    if (EPI == MID_GATED) ((bf16_t*)yv)[i] = from_float<bf16_t>(gate_times_up(a, b));
+    if (EPI == MID_GATED) ((bf16_t*)yv)[i] = from_float<bf16_t>(gate_times_up(gate, a, b));
     else ((TY*)yv)[i] = from_float<TY>(a);
 }
 
@@ -405,7 +408,7 @@ static int launch_mid(const MidArgs& a, const MidPlan& plan, bool finish, hipStr
     if (tqk_check_launch("tqk_mid product")) return -1;
     if (plan.splits > 1 && finish) {
         const size_t total = (size_t)a.M * (EPI == MID_GATED ? a.N / 2 : a.N);
-        mid_finish_kernel<EPI, TY><<<(unsigned)((total + 255) / 256), 256, 0, s>>>(a.partial, a.y, plan.splits, a.M, a.N);
+        mid_finish_kernel<EPI, TY><<<(unsigned)((total + 255) / 256), 256, 0, s>>>(a.partial, a.y, plan.splits, a.M, a.N, Gate{a.gate, a.gate_limit, a.gate_alpha});
         return tqk_check_launch("tqk_mid finish");
     }
     return 0;
@@ -440,7 +443,7 @@ static int check_mid(const MidArgs& a, const void* scratch, bool gated, bool fin
  * (for tqk_add_rmsnorm_sums) and y is not written. */
 extern "C" int tqk_mid_store(const void* x, const void* w_packed, void* y, int y_dtype, int M, int N, int K,
                              void* scratch, int finish, void* stream) {
-    MidArgs a = {(const bf16_t*)x, (const bf16_t*)w_packed, y, (float*)scratch, M, N, K, 0};
+    MidArgs a = {(const bf16_t*)x, (const bf16_t*)w_packed, y, (float*)scratch, M, N, K, 0, 0, 0.f, 1.f};
     if (check_mid(a, scratch, false, finish != 0, "tqk_mid_store")) return -1;
     TQK_REQUIRE(y_dtype == TQK_F32 || y_dtype == TQK_BF16, "tqk_mid_store: unknown output dtype %d", y_dtype);
     if (M == 0) return 0;
@@ -453,7 +456,14 @@ extern "C" int tqk_mid_store(const void* x, const void* w_packed, void* y, int y
 
 /* y[M, N/2] = silu(gate) * up, w = gate rows then up rows, packed in two parts. */
 extern "C" int tqk_mid_gated(const void* x, const void* w_packed, void* y, int M, int N, int K, void* scratch, void* stream) {
-    MidArgs a = {(const bf16_t*)x, (const bf16_t*)w_packed, y, (float*)scratch, M, N, K, 0};
+    return tqk_mid_gated_act(x, w_packed, y, M, N, K, scratch, TQK_GATE_SILU, 0.f, 1.f, stream);
+}
+
+/* the same with another gate (TQK_GATE_*: common.h) */
+extern "C" int tqk_mid_gated_act(const void* x, const void* w_packed, void* y, int M, int N, int K, void* scratch, int gate, float limit,
+                                 float alpha, void* stream) {
+    TQK_REQUIRE(gate >= 0 && gate < TQK_GATE_KINDS, "tqk_mid_gated: unknown gate %d", gate);
+    MidArgs a = {(const bf16_t*)x, (const bf16_t*)w_packed, y, (float*)scratch, M, N, K, 0, gate, limit, alpha};
     if (check_mid(a, scratch, true, true, "tqk_mid_gated")) return -1;
     if (M == 0) return 0;
     const MidPlan plan = mid_plan(N, K, true);

@@ -78,6 +78,8 @@ struct FusedArgs {
     int M, N, K;
     // store / gated
     void* y;
+    int gate;                   // gated: which gate (TQK_GATE_*), with its limit and alpha
+    float gate_limit, gate_alpha;
     // residual
     float* h;                   // [M, N]
     const bf16_t* next_norm_w;  // [N] weight of the norm that follows, or null
@@ -319,7 +321,7 @@ void skinny_fused_kernel(const FusedArgs p) {
             if (n >= n_out) continue;
             const float g = to_float(from_float<bf16_t>(acc[0][r] * inv_rms));
             const float up = to_float(from_float<bf16_t>(acc[1][r] * inv_rms));
-            y[(size_t)m * n_out + n] = from_float<bf16_t>((g / (1.f + expf(-g))) * up);
+            y[(size_t)m * n_out + n] = from_float<bf16_t>(gate_value(p.gate, p.gate_limit, p.gate_alpha, g, up));
         }
     } else if constexpr (EPI == EPI_RESIDUAL) {
         float sq = 0.f;
@@ -469,7 +471,15 @@ extern "C" int tqk_fused_store(const void* x, const int32_t* x_rows, const float
 /* y[M, N/2] = silu(gate) * up of the (normalised) product, w = gate rows then up rows. */
 extern "C" int tqk_fused_gated(const void* x, const float* ss_parts, int n_ss_parts, float eps, const void* w, int w_packed, void* y,
                                int M, int N, int K, void* stream) {
+    return tqk_fused_gated_act(x, ss_parts, n_ss_parts, eps, w, w_packed, y, M, N, K, TQK_GATE_SILU, 0.f, 1.f, stream);
+}
+
+/* the same with another gate (TQK_GATE_*: common.h) */
+extern "C" int tqk_fused_gated_act(const void* x, const float* ss_parts, int n_ss_parts, float eps, const void* w, int w_packed, void* y,
+                                   int M, int N, int K, int gate, float limit, float alpha, void* stream) {
+    TQK_REQUIRE(gate >= 0 && gate < TQK_GATE_KINDS, "tqk_fused_gated: unknown gate %d", gate);
     FusedArgs a = {};
+    a.gate = gate; a.gate_limit = limit; a.gate_alpha = alpha;
     a.x = (const bf16_t*)x; a.ss_parts = ss_parts; a.n_ss_parts = n_ss_parts; a.eps = eps; a.w = (const bf16_t*)w; a.w_packed = w_packed;
     a.M = M; a.N = N; a.K = K; a.y = y;
     if (check_common(a, "tqk_fused_gated")) return -1;

@@ -175,6 +175,61 @@ int tqk_attention_prefill(const void* q, const void* keys, const void* values, c
 /* out[t, i] = silu(gate_up[t, i]) * gate_up[t, inter + i] */
 int tqk_swiglu(const void* gate_up, void* out, int act_dtype, int n_tokens, int inter, void* stream);
 
+/* Gates of feed-forwards other than SiLU.  gate: 0 g sigmoid(g) u; 1 max(g, 0) u; 2 g' sigmoid(alpha g') (u' + 1) with
+ * g' = min(g, limit) and u' = clamp(u, -limit, limit); 3 gelu_tanh(g) u.  tqk_gated_act is tqk_swiglu, and
+ * tqk_fused_gated_act and tqk_mid_gated_act are tqk_fused_gated and tqk_mid_gated, with the gate named. */
+int tqk_gated_act(const void* gate_up, void* out, int act_dtype, int n_tokens, int inter, int gate, float limit, float alpha,
+                  void* stream);
+int tqk_fused_gated_act(const void* x, const float* ss_parts, int n_ss_parts, float eps, const void* w, int w_packed, void* y,
+                        int M, int N, int K, int gate, float limit, float alpha, void* stream);
+int tqk_mid_gated_act(const void* x, const void* w_packed, void* y, int M, int N, int K, void* scratch, int gate, float limit,
+                      float alpha, void* stream);
+
+/* Attention through a low-rank latent (latent.hip).  Every position leaves one cache row [rk + dr]: the normed
+ * latent and one rotated key part, shared by all heads; pages are [n_pages][64][rk + dr].
+ * tqk_latent_split: row t of proj (row_stride values) begins [q_rank | kv_rank + rot_dim (absent when kv_rank == 0) | n_gate].  cq_out
+ * [tokens, q_rank] = RMS norm of the first part times q_norm_w; the second part goes into the cache row of the token's
+ * position (RMS norm times kv_norm_w of its first kv_rank values, rotation in halves of the first rot_dims of the
+ * others by the angle table row tok_pos[t]); gate_out [tokens, n_gate] = sigmoid of the last part, float32. */
+int tqk_latent_max_rank(void);          /* the largest latent (rk) tqk_latent_attention takes */
+int tqk_latent_max_row(void);           /* the largest cache row (rk + dr) it takes */
+int tqk_latent_split(const void* proj, int act_dtype, int row_stride, int q_rank, int kv_rank, int rot_dim, int n_gate, const void* q_norm_w,
+                     const void* kv_norm_w, int norm_dtype, float eps, const float* cos_table, const float* sin_table,
+                     int rot_dims, int max_positions, const int32_t* tok_seq, const int32_t* tok_pos,
+                     const int32_t* page_table, int table_width, void* cache, int n_pages, void* cq_out, float* gate_out,
+                     int n_tokens, void* stream);
+/* qa [tokens, heads, rk + dr] float32: qa[:rk] = W_uk,h^T q[:dn] (w_uk [heads * dn, rk]), qa[rk:] = q[dn:] rotated */
+int tqk_latent_absorb(const void* q, int act_dtype, const void* w_uk, int w_dtype, int n_heads, int dn, int dr, int rk,
+                      const float* cos_table, const float* sin_table, int rot_dims, int max_positions,
+                      const int32_t* tok_pos, float* qa, int n_tokens, void* stream);
+/* out [tokens, heads, rk] float32 = softmax over the visible positions of (qa . row) * scale, times row[:rk];
+ * visible: lo..tok_pos[t], lo = max(0, tok_pos - window + 1) if window > 0 else 0 */
+int tqk_latent_attention(const float* qa, const void* cache, int cache_dtype, const int32_t* tok_seq, const int32_t* tok_pos,
+                         const int32_t* page_table, int table_width, int n_seqs, int n_pages, int window, float scale,
+                         float* out, int n_tokens, int n_heads, int rk, int dr, void* stream);
+/* y [tokens, heads * dv] = gate[t, h] * W_uv,h o[t, h] (w_uv [heads * dv, rk]; gate may be null) */
+int tqk_latent_values(const float* o, const void* w_uv, int w_dtype, const float* gate, int n_heads, int rk, int dv, void* y,
+                      int y_dtype, int n_tokens, void* stream);
+
+/* A feed-forward of routed experts (moe.hip).  tqk_moe_route: idx, weight [tokens, top]: the `top` experts with the
+ * largest softmax(W_r x) and that score times scale.  tqk_moe_group: pair p = (token, choice) gets row pair_pos[p]
+ * among its expert's rows, sorted_tok[row] names the row's token; tile lists of tqk_moe_max_tiles(pairs, experts)
+ * entries and their number *n_tiles, all on the device.  tqk_moe_product: rows (x[x_rows[row]] or x[row]) of every
+ * tile times its expert's weight (w + expert * expert_stride: [N, K], gated: gate rows then up rows [2 N, K]) into
+ * y [pairs, N].  tqk_moe_combine: out[t] = sum_k weight[t, k] y[pair_pos[t, k]] + shared[t] (shared may be null). */
+int tqk_moe_max_experts(void);
+int tqk_moe_tile_rows(void);
+int tqk_moe_max_tiles(int n_pairs, int n_experts);
+int tqk_moe_route(const void* x, int act_dtype, const void* w_router, int w_dtype, int n_experts, int hidden, int top, float scale,
+                  int32_t* idx, float* weight, int n_tokens, void* stream);
+int tqk_moe_group(const int32_t* idx, int n_tokens, int top, int n_experts, int32_t* pair_pos, int32_t* sorted_tok,
+                  int32_t* tile_expert, int32_t* tile_row0, int32_t* tile_rows, int32_t* n_tiles, void* stream);
+int tqk_moe_product(const void* x, int act_dtype, const int32_t* x_rows, const void* w, int w_dtype, long long expert_stride, void* y,
+                    int N, int K, int gated, int gate, float limit, float alpha, const int32_t* tile_expert,
+                    const int32_t* tile_row0, const int32_t* tile_rows, const int32_t* n_tiles, int max_tiles, void* stream);
+int tqk_moe_combine(const void* y, int act_dtype, const int32_t* pair_pos, const float* weight, int top, const void* shared, void* out,
+                    int n_tokens, int hidden, void* stream);
+
 /* out[r] = lowest index of the largest value of logits[r, :]; scratch: at least
  * tqk_argmax_scratch_floats(n_rows, vocab) floats of device memory. */
 int tqk_argmax_scratch_floats(int n_rows, int vocab);

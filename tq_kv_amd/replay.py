@@ -37,8 +37,11 @@ def main(argv=None):
 
     os.makedirs(args.out, exist_ok=True)
     model = Model.from_dir(args.model, dtype=args.dtype, device="cuda")
-    max_tokens = max(PAGE, (args.max_tokens + PAGE - 1) // PAGE * PAGE)
-    engine = Engine(model, max_tokens=max_tokens, max_slots=max_tokens // PAGE)
+    # every live request may end in a page that is partly used, and a request may be as short as one token: room for
+    # the tokens in whole pages plus a page for each of some hundred requests
+    slots = 256
+    max_tokens = max(PAGE, (args.max_tokens + PAGE - 1) // PAGE * PAGE) + slots * PAGE
+    engine = Engine(model, max_tokens=max_tokens, max_slots=max(slots, args.max_tokens // PAGE))
     slots = {}
     for line in sys.stdin:
         line = line.strip()

@@ -14,6 +14,11 @@ peak and (`*_of_probe`) against the probe.
 The reference measures tokens per second of one chat request including its prompt
 (src/main.rs:1123-1143); here decoding is timed alone, the prompt pass is reported beside it, and the
 reference's prompt-inclusive figure goes into `end_to_end_tok_per_s`.
+
+`python bench.py --latent` is another measurement with a line of its own (the default workload above is untouched): the
+Nikasun design (attention through cached latents with a window, routed experts) at a few sizes that resemble a real
+model's layers, beside a Qwen2 shape of the same width, depth, heads and active feed-forward size: prompt pass and
+decoding of both, tokens a second.
 """
 import argparse
 import gc
@@ -39,6 +44,8 @@ def main():
     ap.add_argument("--no-long", action="store_true", help="skip the points at 8192 tokens of context")
     ap.add_argument("--no-tune", action="store_true", help="do not let the matrix library try its kernels for the prompt's size")
     ap.add_argument("--no-probe", action="store_true")
+    ap.add_argument("--latent", action="store_true", help="measure the Nikasun design beside a Qwen2 shape of equal size instead of the default workload")
+    ap.add_argument("--latent-sizes", default="2048,4096", help="widths of the --latent comparison")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this library runs on one GPU; --gpus %d is not supported" % args.gpus)
@@ -140,6 +147,10 @@ def main():
     def release():
         gc.collect()
         torch.cuda.empty_cache()
+
+    # -- another design beside the closest existing one -----------------------------------------------
+    if args.latent:
+        return latent_comparison(args, torch, Model, Engine, note, timed_prefill, decode, random_prompts, release)
 
     # -- the headline shape -------------------------------------------------------------------------
     raw = dict(catalog.find(args.shape))
@@ -270,6 +281,65 @@ def main():
         "end_to_end_tok_per_s": round(end_to_end, 1),
     }
     print(json.dumps(line))
+    return 0
+
+
+def latent_shapes(width, layers=4):
+    """A Nikasun configuration and a Qwen2 one of the same width, depth, heads, head size and active feed-forward size."""
+    heads, dim = width // 128, 128
+    experts, top, ff = (32, 4, width // 2) if width <= 2048 else (64, 6, width // 4)
+    shared = 2 * ff
+    active = top * ff + shared
+    mixer = {"heads": heads, "dim": dim, "rot_dim": 64, "vdim": dim, "q_rank": 3 * width // 8, "kv_rank": 512, "scale": (dim + 64) ** -0.5,
+             "rot": {"base": 10000.0, "dims": 64}, "mask": {"size": 1024}}
+    moe = {"kind": "moe", "router": {"experts": experts, "top": top, "scale": 1.0}, "expert": {"ff": ff, "limit": 7.0},
+           "shared": {"ff": shared, "limit": 7.0}}
+    lay = []
+    for l in range(layers):
+        m = dict(mixer)
+        if l % 2 == 1:
+            m["kv_from"] = l - 1
+        lay.append({"type": "latent_attention", "mixer": m, "mlp": {"kind": "dense", "ff": active} if l == 0 else moe})
+    nikasun = {"architecture": "Nikasun", "vocab": 32000, "width": width, "embedding": {"scale": width ** 0.5}, "norm": {"eps": 1e-5},
+               "layers": lay, "max_positions": 8192}
+    qwen2 = {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "hidden_act": "silu", "vocab_size": 32000, "hidden_size": width,
+             "intermediate_size": active, "num_hidden_layers": layers, "num_attention_heads": heads, "num_key_value_heads": max(1, heads // 4),
+             "head_dim": dim, "rms_norm_eps": 1e-5, "rope_theta": 10000.0, "max_position_embeddings": 8192, "tie_word_embeddings": True,
+             "use_sliding_window": True, "sliding_window": 1024, "max_window_layers": 0}
+    return nikasun, qwen2, {"width": width, "layers": layers, "heads": heads, "experts": experts, "top": top, "expert_ff": ff,
+                            "shared_ff": shared, "active_ff": active, "q_rank": mixer["q_rank"], "kv_rank": 512, "window": 1024}
+
+
+def latent_comparison(args, torch, Model, Engine, note, timed_prefill, decode, random_prompts, release):
+    prompt_len, out = 2048, {}
+    for width in [int(x) for x in args.latent_sizes.split(",")]:
+        nikasun, qwen2, sizes = latent_shapes(width)
+        row = {"sizes": sizes}
+        for name, raw in (("nikasun", nikasun), ("qwen2", qwen2)):
+            note("width %d, %s: random weights" % (width, name))
+            model = Model.random(raw, seed=0, dtype="bfloat16", device="cuda:0")
+            engine = Engine(model, max_tokens=64 * (prompt_len + 256))
+            if not args.no_tune:
+                model.tune_library(prompt_len)
+            times = timed_prefill(engine, random_prompts(32000, [prompt_len]), 5)[2:]
+            row[name + "_prefill_tok_s"] = round(prompt_len / statistics.median(times), 1)
+            row[name + "_prefill_ms"] = round(statistics.median(times) * 1e3, 3)
+            for batch in (8, 64):
+                note("width %d, %s: decode at batch %d" % (width, name, batch))
+                tps, sec, _ = decode(engine, random_prompts(32000, [prompt_len] * batch), min(args.steps, 32), 4)
+                row["%s_decode_b%d_tok_s" % (name, batch)] = round(tps, 1)
+                row["%s_decode_b%d_ms" % (name, batch)] = round(sec * 1e3, 4)
+            engine = model = None
+            release()
+        for key in ("prefill_tok_s", "decode_b8_tok_s", "decode_b64_tok_s"):
+            row["ratio_" + key] = round(row["nikasun_" + key] / row["qwen2_" + key], 3)
+        out["width_%d" % width] = row
+    first = out["width_%d" % int(args.latent_sizes.split(",")[0])]
+    print(json.dumps({"metric": "decode tok/s @ batch 8, Nikasun design at width %s" % args.latent_sizes.split(",")[0],
+                      "value": first["nikasun_decode_b8_tok_s"], "unit": "tokens/s", "n_gpus": 1, "steps": min(args.steps, 32), "warmup": 4,
+                      "ms_per_step": first["nikasun_decode_b8_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+                      "dtype": "bf16", "data": "synthetic", "config": {"model": "nikasun beside qwen2 at equal size", "prompt_len": prompt_len,
+                                                                     "weights": "random"}, "comparison": out}))
     return 0
 
 

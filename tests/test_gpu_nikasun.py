@@ -164,7 +164,7 @@ def test_latent_attention_part(dtype, shape):
     reader = env.build("mixer", latent_spec(m2, hidden, eps, own=False))
     assert att.cache_need() == reader.cache_need() and att.graph_safe
     assert "dkv" in att.tensors() and "dkv" not in reader.tensors()
-    gain = {"uq": 3.0, "uk": 3.0, "g": 2.0}
+    gain = {"uq": 2.0, "uk": 2.0, "g": 2.0}
     w, w2 = load(att, rand_weights(att, 4, gain), dtype), load(reader, rand_weights(reader, 5, gain), dtype)
     cache = Cache([att.cache_need(), reader.cache_need()], [None, 0], 64 * 16, 4, DT[dtype], DEV)
     xs = [torch.randn(n, hidden).to(DT[dtype]) for n in (150, 40)]
@@ -224,7 +224,7 @@ def run_cut(eng, toks, cuts, want_all=True):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name,sharp", [("mixed", 1.0), ("mixed", 3.0), ("ones", 1.0), ("odd", 2.0)])
+@pytest.mark.parametrize("name,sharp", [("mixed", 1.0), ("mixed", 2.0), ("ones", 1.0), ("odd", 2.0)])
 def test_whole_prompts_and_every_cut(name, sharp, dtype, tmp_path_factory):
     cfg, w, eng = engine(name, dtype, tmp_path_factory, sharp)
     assert eng.model.spec.architecture == "Nikasun" and eng.model.graph_safe
@@ -242,7 +242,7 @@ def test_whole_prompts_and_every_cut(name, sharp, dtype, tmp_path_factory):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_batches_of_unequal_requests_and_reused_slots(dtype, tmp_path_factory):
-    cfg, w, eng = engine("mixed", dtype, tmp_path_factory, 3.0, max_tokens=64 * 12, slots=4)
+    cfg, w, eng = engine("mixed", dtype, tmp_path_factory, 2.0, max_tokens=64 * 12, slots=4)
     reqs = [N.tokens(n, cfg["vocab"], 30 + n) for n in (130, 7, 66, 1, 95, 64, 20)]
     want = [N.plain_logits(cfg, w, t) for t in reqs]
     alone = [run_cut(eng, t, []) for t in reqs]
@@ -284,6 +284,7 @@ def poison(eng):
         free = [p for p in range(g.pool.n) if p not in held]
         if free:
             g.keys[:, torch.tensor(free, device=g.keys.device)] = float("nan")
+            g.values[:, torch.tensor(free, device=g.keys.device)] = float("nan")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

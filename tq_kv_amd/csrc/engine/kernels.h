@@ -52,15 +52,21 @@ TQ_KERNEL(fused_gated_act, cptr, cf32, int, float, cptr, int, void*, int, int, i
 TQ_KERNEL(mid_gated_act, cptr, cptr, void*, int, int, int, void*, int, float, float, void*);
 TQ_QUERY(int, latent_max_rank);
 TQ_QUERY(int, latent_max_row);
-TQ_KERNEL(latent_split, cptr, int, int, int, int, int, int, cptr, cptr, int, float, cf32, cf32, int, int, ci32, ci32, ci32, int, void*, int, void*,
-          float*, int, void*);
-TQ_KERNEL(latent_absorb, cptr, int, cptr, int, int, int, int, int, cf32, cf32, int, int, ci32, float*, int, void*);
+TQ_KERNEL(latent_split, cptr, int, int, int, int, int, int, cptr, cptr, int, float, cf32, cf32, int, int, ci32, ci32, ci32, int, void*, void*, int,
+          void*, float*, int, void*);
+TQ_QUERY(int, latent_attention_mfma_supported, int, int);
+TQ_KERNEL(latent_attention_mfma, cf32, cptr, cptr, ci32, ci32, ci32, int, int, int, int, float, float*, int, int, int, int, void*);
+TQ_KERNEL(latent_absorb, cptr, int, cptr, int, int, int, int, int, cf32, cf32, int, int, ci32, float*, int, int, void*);
 TQ_KERNEL(latent_attention, cf32, cptr, int, ci32, ci32, ci32, int, int, int, int, float, float*, int, int, int, int, void*);
 TQ_KERNEL(latent_values, cf32, cptr, int, cf32, int, int, int, void*, int, int, void*);
 TQ_QUERY(int, moe_max_experts);
-TQ_QUERY(int, moe_max_tiles, int, int);
+TQ_QUERY(int, moe_max_tiles, int, int, int);
+TQ_QUERY(int, moe_tile_rows);
+TQ_QUERY(int, grouped_supported, int);
+TQ_KERNEL(moe_product_mfma, cptr, ci32, cptr, long long, void*, int, int, int, int, float, float, ci32, ci32, ci32, ci32, int, int, void*);
+TQ_KERNEL(head_product, cptr, int, long long, long long, cptr, void*, int, long long, long long, cf32, int, int, int, int, void*);
 TQ_KERNEL(moe_route, cptr, int, cptr, int, int, int, int, float, int32_t*, float*, int, void*);
-TQ_KERNEL(moe_group, ci32, int, int, int, int32_t*, int32_t*, int32_t*, int32_t*, int32_t*, int32_t*, void*);
+TQ_KERNEL(moe_group, ci32, int, int, int, int, int32_t*, int32_t*, int32_t*, int32_t*, int32_t*, int32_t*, void*);
 TQ_KERNEL(moe_product, cptr, int, ci32, cptr, int, long long, void*, int, int, int, int, float, float, ci32, ci32, ci32, ci32, int, void*);
 TQ_KERNEL(moe_combine, cptr, int, ci32, cf32, int, cptr, void*, int, int, void*);
 TQ_QUERY(int, argmax_scratch_floats, int, int);

@@ -105,12 +105,26 @@ public:
         w_uq_ = make_weight(take(t, "uq"), 1, false, stream);
         uk_ = take(t, "uk");
         uv_ = take(t, "uv");
+        // For the matrix cores a head's W_uk is wanted with the latent's elements as its rows, [heads][kv_rank][head_dim]:
+        // turned once, on the host.
+        if (uk_->t.dtype == BF16 && uv_->t.dtype == BF16 && dn_ % 8 == 0 && (dn_ + dr_) % 8 == 0 && kv_rank_ % 8 == 0) {
+            std::vector<uint16_t> rows((size_t)uk_->t.numel()), turned(rows.size());
+            copy_to_host(rows.data(), uk_->t.data, uk_->t.bytes(), stream);
+            for (int h = 0; h < n_heads_; ++h)
+                for (int d = 0; d < dn_; ++d)
+                    for (int j = 0; j < kv_rank_; ++j)
+                        turned[((size_t)h * kv_rank_ + j) * dn_ + d] = rows[((size_t)h * dn_ + d) * kv_rank_ + j];
+            uk_turned_ = make_owned(BF16, {n_heads_, kv_rank_, dn_});
+            copy_to_device(uk_turned_->t.data, turned.data(), turned.size() * 2, stream);
+            stream_synchronize(stream);
+        }
         w_o_ = make_weight(take(t, "o"), 1, false, stream);
     }
     OwnedPtr held(const std::string& name) const override {
         if (name == "in.weight") return w_in_.rows;
         if (name == "uq") return w_uq_.rows;
         if (name == "uk") return uk_;
+        if (name == "uk.turned") return uk_turned_;
         if (name == "uv") return uv_;
         if (name == "o") return w_o_.rows;
         if (name == "dq.norm") return q_norm_;
@@ -128,7 +142,7 @@ public:
         CacheNeed n;
         n.kind = CacheNeed::Pages;
         n.key_page = {TQE_PAGE, kv_rank_ + dr_};
-        n.value_page = {1};                     // values are the rows' first kv_rank elements: nothing of their own is kept
+        n.value_page = {kv_rank_, TQE_PAGE};    // the latents a second time, turned, for the matrix cores (bfloat16 runs)
         n.window = cache_window_;
         return n;
     }
@@ -151,22 +165,39 @@ public:
         const float* sin = turns ? (const float*)tb.sin.data : nullptr;
         const int rot_dims = turns ? tb.rot_dim : 0, max_pos = turns ? (int)tb.cos.shape[0] : 0;
 
+        // a bfloat16 cache is read by the matrix cores, which want the latents a second time, turned
+        const bool on_cores = entry.keys.dtype == BF16 && policy().prefill_mfma && policy().decode_mfma &&
+                              K::latent_attention_mfma_supported.raw(kv_rank_, dr_) != 0;
         Tensor first = linear(c, x.x, w_in_, nullptr, dtype).t;                 // [n, in_cols_]
         Tensor cq = c.alloc(dtype, {n, q_rank_});
         Tensor gate = gated_ ? c.alloc(F32, {n, n_heads_}) : Tensor();
         K::latent_split(first.data, dtype, (int)in_cols_, q_rank_, own_kv_ ? kv_rank_ : 0, dr_, gated_ ? n_heads_ : 0, q_norm_->t.data,
                         kv_norm_ ? kv_norm_->t.data : nullptr, q_norm_->t.dtype, eps_, cos, sin, rot_dims, max_pos, c.dev.tok_seq, c.dev.tok_pos,
-                        table.dev, table.width, own_kv_ ? entry.keys.data : nullptr, n_pages, cq.data, (float*)gate.data, (int)n, c.stream);
+                        table.dev, table.width, own_kv_ ? entry.keys.data : nullptr, own_kv_ && on_cores ? entry.values.data : nullptr, n_pages, cq.data,
+                        (float*)gate.data, (int)n, c.stream);
         Tensor q = linear(c, cq, w_uq_, nullptr, dtype).t;                        // [n, heads, dn + dr]
         Tensor qa = c.alloc(F32, {n, n_heads_, kv_rank_ + dr_});
+        // the two products per head: bfloat16 on the matrix cores where the sizes allow, else in the latent kernels themselves
+        const bool heads_on_cores = dtype == BF16 && uk_turned_ && policy().skinny;
+        if (heads_on_cores)
+            K::head_product(q.data, 0, (long long)n_heads_ * (dn_ + dr_), (long long)(dn_ + dr_), uk_turned_->t.data, qa.data, 1,
+                            (long long)n_heads_ * (kv_rank_ + dr_), (long long)(kv_rank_ + dr_), nullptr, (int)n, n_heads_, kv_rank_, dn_, c.stream);
         K::latent_absorb(q.data, dtype, uk_->t.data, uk_->t.dtype, n_heads_, dn_, dr_, kv_rank_, cos, sin, rot_dims, max_pos, c.dev.tok_pos,
-                         (float*)qa.data, (int)n, c.stream);
+                         (float*)qa.data, (int)n, heads_on_cores ? 1 : 0, c.stream);
         Tensor o = c.alloc(F32, {n, n_heads_, kv_rank_});
-        K::latent_attention((const float*)qa.data, entry.keys.data, entry.keys.dtype, c.dev.tok_seq, c.dev.tok_pos, table.dev, table.width, c.n_seqs,
-                            n_pages, window_, scale_, (float*)o.data, (int)n, n_heads_, kv_rank_, dr_, c.stream);
+        if (on_cores)
+            K::latent_attention_mfma((const float*)qa.data, entry.keys.data, entry.values.data, c.dev.tok_seq, c.dev.tok_pos, table.dev, table.width,
+                                     c.n_seqs, n_pages, window_, scale_, (float*)o.data, (int)n, n_heads_, kv_rank_, dr_, c.stream);
+        else
+            K::latent_attention((const float*)qa.data, entry.keys.data, entry.keys.dtype, c.dev.tok_seq, c.dev.tok_pos, table.dev, table.width, c.n_seqs,
+                                n_pages, window_, scale_, (float*)o.data, (int)n, n_heads_, kv_rank_, dr_, c.stream);
         Tensor y = c.alloc(dtype, {n, (int64_t)n_heads_ * dv_});
-        K::latent_values((const float*)o.data, uv_->t.data, uv_->t.dtype, (const float*)gate.data, n_heads_, kv_rank_, dv_, y.data, dtype, (int)n,
-                         c.stream);
+        if (heads_on_cores)
+            K::head_product(o.data, 1, (long long)n_heads_ * kv_rank_, (long long)kv_rank_, uv_->t.data, y.data, 0, (long long)n_heads_ * dv_,
+                            (long long)dv_, (const float*)gate.data, (int)n, n_heads_, dv_, kv_rank_, c.stream);
+        else
+            K::latent_values((const float*)o.data, uv_->t.data, uv_->t.dtype, (const float*)gate.data, n_heads_, kv_rank_, dv_, y.data, dtype, (int)n,
+                             c.stream);
         if (stream) {
             add_product(c, *stream, y, w_o_);
             return Tensor();
@@ -181,7 +212,7 @@ private:
     bool own_kv_, gated_;
     std::shared_ptr<Position> position_;
     Weight w_in_, w_uq_, w_o_;
-    OwnedPtr q_norm_, kv_norm_, uk_, uv_;
+    OwnedPtr q_norm_, kv_norm_, uk_, uv_, uk_turned_;
 };
 
 }  // namespace

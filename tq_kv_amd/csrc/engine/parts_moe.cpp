@@ -113,7 +113,12 @@ public:
         const int64_t n = x.x.shape[0];
         const int dtype = x.x.dtype;
         const int64_t pairs = n * top_;
-        const int max_tiles = K::moe_max_tiles.raw((int)pairs, n_experts_);
+        // bfloat16 on the matrix cores, in tiles whose size follows the rows an expert gets on average; else the plain kernel
+        const bool on_cores = dtype == BF16 && gate_up_->t.dtype == BF16 && down_->t.dtype == BF16 && policy().skinny && hidden_ % 8 == 0 &&
+                              inter_ % 8 == 0 && K::grouped_supported.raw((int)hidden_) != 0;
+        const int64_t per_expert = pairs / n_experts_;
+        const int tile_m = !on_cores ? K::moe_tile_rows.raw() : per_expert >= 48 ? 64 : per_expert >= 24 ? 32 : 16;
+        const int max_tiles = K::moe_max_tiles.raw((int)pairs, n_experts_, tile_m);
         Tensor idx = c.alloc(I32, {n, top_}), weight = c.alloc(F32, {n, top_});
         Tensor pair_pos = c.alloc(I32, {pairs}), sorted_tok = c.alloc(I32, {pairs});
         Tensor tiles = c.alloc(I32, {3, max_tiles}), n_tiles = c.alloc(I32, {4});
@@ -122,17 +127,25 @@ public:
         int32_t* tile_rows = tile_row0 + max_tiles;
         K::moe_route(x.x.data, dtype, router_->t.data, router_->t.dtype, n_experts_, (int)hidden_, top_, router_scale_, (int32_t*)idx.data,
                      (float*)weight.data, (int)n, c.stream);
-        K::moe_group((const int32_t*)idx.data, (int)n, top_, n_experts_, (int32_t*)pair_pos.data, (int32_t*)sorted_tok.data, tile_expert, tile_row0,
+        K::moe_group((const int32_t*)idx.data, (int)n, top_, n_experts_, tile_m, (int32_t*)pair_pos.data, (int32_t*)sorted_tok.data, tile_expert, tile_row0,
                      tile_rows, (int32_t*)n_tiles.data, c.stream);
         Tensor shared_out;
         if (shared_) shared_out = shared_->forward(c, x, nullptr);
         Tensor act = c.alloc(dtype, {pairs, inter_});
-        K::moe_product(x.x.data, dtype, (const int32_t*)sorted_tok.data, gate_up_->t.data, gate_up_->t.dtype, (long long)(2 * inter_ * hidden_), act.data,
-                       (int)inter_, (int)hidden_, 1, gate_.kind, gate_.limit, gate_.alpha, tile_expert, tile_row0, tile_rows,
-                       (const int32_t*)n_tiles.data, max_tiles, c.stream);
         Tensor y = c.alloc(dtype, {pairs, hidden_});
-        K::moe_product(act.data, dtype, nullptr, down_->t.data, down_->t.dtype, (long long)(hidden_ * inter_), y.data, (int)hidden_, (int)inter_, 0, 0,
-                       0.f, 1.f, tile_expert, tile_row0, tile_rows, (const int32_t*)n_tiles.data, max_tiles, c.stream);
+        if (on_cores) {
+            K::moe_product_mfma(x.x.data, (const int32_t*)sorted_tok.data, gate_up_->t.data, (long long)(2 * inter_ * hidden_), act.data, (int)inter_,
+                                (int)hidden_, 1, gate_.kind, gate_.limit, gate_.alpha, tile_expert, tile_row0, tile_rows,
+                                (const int32_t*)n_tiles.data, max_tiles, tile_m, c.stream);
+            K::moe_product_mfma(act.data, nullptr, down_->t.data, (long long)(hidden_ * inter_), y.data, (int)hidden_, (int)inter_, 0, 0, 0.f, 1.f,
+                                tile_expert, tile_row0, tile_rows, (const int32_t*)n_tiles.data, max_tiles, tile_m, c.stream);
+        } else {
+            K::moe_product(x.x.data, dtype, (const int32_t*)sorted_tok.data, gate_up_->t.data, gate_up_->t.dtype, (long long)(2 * inter_ * hidden_),
+                           act.data, (int)inter_, (int)hidden_, 1, gate_.kind, gate_.limit, gate_.alpha, tile_expert, tile_row0, tile_rows,
+                           (const int32_t*)n_tiles.data, max_tiles, c.stream);
+            K::moe_product(act.data, dtype, nullptr, down_->t.data, down_->t.dtype, (long long)(hidden_ * inter_), y.data, (int)hidden_, (int)inter_, 0,
+                           0, 0.f, 1.f, tile_expert, tile_row0, tile_rows, (const int32_t*)n_tiles.data, max_tiles, c.stream);
+        }
         Tensor out = c.alloc(dtype, {n, hidden_});
         K::moe_combine(y.data, dtype, (const int32_t*)pair_pos.data, (const float*)weight.data, top_, shared_out.data, out.data, (int)n,
                        (int)hidden_, c.stream);

@@ -30,8 +30,8 @@ void latent_split_kernel(const TA* __restrict__ proj, int row_stride, int q_rank
                          const TW* __restrict__ q_norm_w, const TW* __restrict__ kv_norm_w, float eps,
                          const float* __restrict__ cos_table, const float* __restrict__ sin_table, int rot_dims, int max_positions,
                          const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos,
-                         const int32_t* __restrict__ page_table, int table_width, TA* __restrict__ cache, int n_pages,
-                         TA* __restrict__ cq_out, float* __restrict__ gate_out) {
+                         const int32_t* __restrict__ page_table, int table_width, TA* __restrict__ cache, TA* __restrict__ turned,
+                         int n_pages, TA* __restrict__ cq_out, float* __restrict__ gate_out) {
     __shared__ float scratch[8];
     const int t = blockIdx.x;
     const int kv_cols = kv_rank > 0 ? kv_rank + rot_dim : 0;
@@ -57,7 +57,13 @@ void latent_split_kernel(const TA* __restrict__ proj, int row_stride, int q_rank
     const int page = page_table[(size_t)tok_seq[t] * table_width + pos / TQK_PAGE];
     if (page < 0 || page >= n_pages) return;
     TA* dst = cache + ((size_t)page * TQK_PAGE + (size_t)(pos % TQK_PAGE)) * kv_cols;
-    for (int i = threadIdx.x; i < kv_rank; i += blockDim.x) dst[i] = from_float<TA>(to_float(kv[i]) * inv_kv * to_float(kv_norm_w[i]));
+    // the latent a second time, turned: [element][place of the position], for the matrix cores' second product
+    TA* dst_t = turned ? turned + (size_t)page * kv_rank * TQK_PAGE + value_place(pos % TQK_PAGE) : nullptr;
+    for (int i = threadIdx.x; i < kv_rank; i += blockDim.x) {
+        const TA v = from_float<TA>(to_float(kv[i]) * inv_kv * to_float(kv_norm_w[i]));
+        dst[i] = v;
+        if (dst_t) dst_t[(size_t)i * TQK_PAGE] = v;
+    }
     const int half = rot_dims / 2;
     const int p = min(pos, max_positions - 1);
     for (int i = threadIdx.x; i < rot_dim; i += blockDim.x) {
@@ -80,7 +86,7 @@ template <typename TA, typename TW>
 __global__ __launch_bounds__(128)
 void latent_absorb_kernel(const TA* __restrict__ q, const TW* __restrict__ w_uk, int n_heads, int dn, int dr, int rk,
                           const float* __restrict__ cos_table, const float* __restrict__ sin_table, int rot_dims, int max_positions,
-                          const int32_t* __restrict__ tok_pos, float* __restrict__ qa, int n_tokens) {
+                          const int32_t* __restrict__ tok_pos, float* __restrict__ qa, int n_tokens, int tail_only) {
     extern __shared__ float q_lds[];            // [LAT_TT][dn + dr]
     const int head = blockIdx.y, t0 = blockIdx.x * LAT_TT, d = dn + dr;
     const int n_t = min(LAT_TT, n_tokens - t0);
@@ -90,7 +96,7 @@ void latent_absorb_kernel(const TA* __restrict__ q, const TW* __restrict__ w_uk,
     }
     __syncthreads();
     const TW* w = w_uk + (size_t)head * dn * rk;
-    for (int j = threadIdx.x; j < rk; j += blockDim.x) {
+    for (int j = threadIdx.x; j < (tail_only ? 0 : rk); j += blockDim.x) {
         float acc[LAT_TT];
 #pragma unroll
         for (int tt = 0; tt < LAT_TT; ++tt) acc[tt] = 0.f;
@@ -188,6 +194,150 @@ void latent_attention_kernel(const float* __restrict__ qa, const TA* __restrict_
     }
 }
 
+// ---- attention on the matrix cores (bfloat16 cache) -------------------------------------------
+// One wave per (token, 16 heads).  v_mfma_f32_16x16x32_bf16, D[16x16] += A[16x32] B[32x16]:
+//   scores^T[key][head] = row[key][:] . qa^T[:][head]
+//       A = 16 cache rows x 32 of their elements, 16 contiguous bytes per lane straight from the page; B = the heads'
+//       absorbed queries, held in registers for the whole walk.  The lane then holds, for head l%16, keys 4*(l/16)+i.
+//   out^T[element][head] = turned[element][key] . P^T[key][head]
+//       B: the eight keys a lane holds of two groups of 16 are the product's eight k slots, so P never leaves its
+//       registers; A: the turned copy of the latents keeps a page's positions in exactly that order (value_place),
+//       16 contiguous bytes per lane.
+// KS: 32-element steps of a cache row the kernel is built for; NCT: 16-element blocks of the latent.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 lat_bf16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float lat_floatx4_t;
+union lat_pack8 {
+    lat_bf16x8_t v;
+    uint16_t u[8];
+    uint4 q;
+};
+
+template <int KS, int NCT>
+__global__ __launch_bounds__(LAT_WAVES * TQK_WAVE)
+void latent_attention_mfma_kernel(const float* __restrict__ qa, const bf16_t* __restrict__ cache, const bf16_t* __restrict__ turned,
+                                  const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos,
+                                  const int32_t* __restrict__ page_table, int table_width, int window, float scale,
+                                  float* __restrict__ out, int n_tokens, int n_heads, int n_chunks, int rk, int dk) {
+    const int wave = threadIdx.x / TQK_WAVE, lane = threadIdx.x % TQK_WAVE;
+    const int item = blockIdx.x * LAT_WAVES + wave;
+    if (item >= n_tokens * n_chunks) return;
+    const int t = item / n_chunks, head = (item % n_chunks) * 16 + lane % 16;
+    const int g = lane / 16, r16 = lane % 16;
+    const int pos = tok_pos[t];
+    const int32_t* pages = page_table + (size_t)tok_seq[t] * table_width;
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int ks_used = (dk + 31) / 32, ct_used = (rk + 15) / 16;
+
+    lat_pack8 bq[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        const int e0 = 32 * ks + 8 * g;
+        bq[ks].q = make_uint4(0, 0, 0, 0);
+        if (head < n_heads && e0 + 8 <= dk) {
+            const float4* src = reinterpret_cast<const float4*>(qa + ((size_t)t * n_heads + head) * dk + e0);
+            const float4 a = src[0], b = src[1];
+            bq[ks].u[0] = float_to_bf16_bits(a.x); bq[ks].u[1] = float_to_bf16_bits(a.y);
+            bq[ks].u[2] = float_to_bf16_bits(a.z); bq[ks].u[3] = float_to_bf16_bits(a.w);
+            bq[ks].u[4] = float_to_bf16_bits(b.x); bq[ks].u[5] = float_to_bf16_bits(b.y);
+            bq[ks].u[6] = float_to_bf16_bits(b.z); bq[ks].u[7] = float_to_bf16_bits(b.w);
+        }
+    }
+    lat_floatx4_t o[NCT];
+#pragma unroll
+    for (int ct = 0; ct < NCT; ++ct) o[ct] = lat_floatx4_t{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+
+    for (int kb = (lo / TQK_PAGE) * TQK_PAGE; kb <= pos; kb += TQK_PAGE) {
+        const int page = max(0, pages[kb / TQK_PAGE]);
+        const bf16_t* kp = cache + (size_t)page * TQK_PAGE * dk;
+        const bf16_t* vp = turned + (size_t)page * rk * TQK_PAGE;
+        lat_floatx4_t s[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) s[j] = lat_floatx4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            if (ks < ks_used) {
+                const int e0 = 32 * ks + 8 * g;
+                const bool in = e0 + 8 <= dk;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    lat_pack8 a;
+                    a.q = in ? *reinterpret_cast<const uint4*>(kp + (size_t)(16 * j + r16) * dk + e0) : make_uint4(0, 0, 0, 0);
+                    s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, bq[ks].v, s[j], 0, 0, 0);
+                }
+            }
+        }
+        // the lane's 16 scores belong to its head and keys kb + 16 j + 4 g + i
+        float p[4][4];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int key = kb + 16 * j + 4 * g + i;
+                const bool valid = key >= lo && key <= pos;
+                p[j][i] = valid ? s[j][i] * scale : -INFINITY;
+                mx = fmaxf(mx, p[j][i]);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, TQK_WAVE));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, TQK_WAVE));
+        const float m_new = fmaxf(m, mx);               // finite: the page holds at least one visible key
+        const float alpha = expf(m - m_new);
+        float sum = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                p[j][i] = expf(p[j][i] - m_new);        // exp(-inf) = 0 for keys that are not seen
+                sum += p[j][i];
+            }
+        sum += __shfl_xor(sum, 16, TQK_WAVE);
+        sum += __shfl_xor(sum, 32, TQK_WAVE);
+        l = l * alpha + sum;
+        m = m_new;
+        lat_pack8 pb[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) pb[h].u[e] = float_to_bf16_bits(p[2 * h + e / 4][e % 4]);
+        // what lies at places of keys that are not seen may be anything: it is replaced by zero
+        const bool edge = kb < lo || kb + TQK_PAGE - 1 > pos;
+#pragma unroll
+        for (int ct = 0; ct < NCT; ++ct) {
+            if (ct < ct_used) {
+                const int col = 16 * ct + r16;
+                o[ct] *= alpha;
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    lat_pack8 a;
+                    a.q = col < rk ? *reinterpret_cast<const uint4*>(vp + (size_t)col * TQK_PAGE + 32 * h + 8 * g) : make_uint4(0, 0, 0, 0);
+                    if (edge) {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            const int key = kb + value_position(32 * h + 8 * g + e);
+                            if (key < lo || key > pos) a.u[e] = 0;
+                        }
+                    }
+                    o[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pb[h].v, o[ct], 0, 0, 0);
+                }
+            }
+        }
+    }
+    if (head >= n_heads) return;
+    float* dst = out + ((size_t)t * n_heads + head) * rk;
+    const float inv = 1.f / l;
+#pragma unroll
+    for (int ct = 0; ct < NCT; ++ct) {
+        if (ct < ct_used) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int col = 16 * ct + 4 * g + i;
+                if (col < rk) dst[col] = o[ct][i] * inv;
+            }
+        }
+    }
+}
+
 // ---- values ----------------------------------------------------------------------------------
 // A block: LAT_TT tokens of one head; a wave takes value columns in turn, its lanes share a row of
 // W_uv (contiguous loads) and their partial sums are added up in a fixed order.
@@ -234,8 +384,8 @@ extern "C" int tqk_latent_max_row(void) { return LAT_MAX_DK; }
 extern "C" int tqk_latent_split(const void* proj, int act_dtype, int row_stride, int q_rank, int kv_rank, int rot_dim, int n_gate, const void* q_norm_w,
                                 const void* kv_norm_w, int norm_dtype, float eps, const float* cos_table, const float* sin_table,
                                 int rot_dims, int max_positions, const int32_t* tok_seq, const int32_t* tok_pos,
-                                const int32_t* page_table, int table_width, void* cache, int n_pages, void* cq_out, float* gate_out,
-                                int n_tokens, void* stream) {
+                                const int32_t* page_table, int table_width, void* cache, void* turned, int n_pages, void* cq_out,
+                                float* gate_out, int n_tokens, void* stream) {
     TQK_REQUIRE(proj && q_norm_w && cq_out, "tqk_latent_split: null pointer");
     TQK_REQUIRE(q_rank > 0 && kv_rank >= 0 && rot_dim >= 0 && n_gate >= 0 && n_tokens >= 0, "tqk_latent_split: bad sizes");
     TQK_REQUIRE(n_gate == 0 || gate_out, "tqk_latent_split: no place for the gates");
@@ -250,8 +400,8 @@ extern "C" int tqk_latent_split(const void* proj, int act_dtype, int row_stride,
 #define TQK_SPLIT(TA, TW)                                                                                                              \
     latent_split_kernel<TA, TW><<<n_tokens, 256, 0, s>>>((const TA*)proj, row_stride, q_rank, kv_rank, rot_dim, n_gate, (const TW*)q_norm_w,       \
                                                          (const TW*)kv_norm_w, eps, cos_table, sin_table, rot_dims, max_positions,     \
-                                                         tok_seq, tok_pos, page_table, table_width, (TA*)cache, n_pages, (TA*)cq_out,  \
-                                                         gate_out)
+                                                         tok_seq, tok_pos, page_table, table_width, (TA*)cache, (TA*)turned, n_pages,  \
+                                                         (TA*)cq_out, gate_out)
     if (act_dtype == TQK_F32 && norm_dtype == TQK_F32) TQK_SPLIT(float, float);
     else if (act_dtype == TQK_F32 && norm_dtype == TQK_BF16) TQK_SPLIT(float, bf16_t);
     else if (act_dtype == TQK_BF16 && norm_dtype == TQK_F32) TQK_SPLIT(bf16_t, float);
@@ -263,8 +413,8 @@ extern "C" int tqk_latent_split(const void* proj, int act_dtype, int row_stride,
 
 extern "C" int tqk_latent_absorb(const void* q, int act_dtype, const void* w_uk, int w_dtype, int n_heads, int dn, int dr, int rk,
                                  const float* cos_table, const float* sin_table, int rot_dims, int max_positions,
-                                 const int32_t* tok_pos, float* qa, int n_tokens, void* stream) {
-    TQK_REQUIRE(q && w_uk && qa && tok_pos, "tqk_latent_absorb: null pointer");
+                                 const int32_t* tok_pos, float* qa, int n_tokens, int tail_only, void* stream) {
+    TQK_REQUIRE(q && (w_uk || tail_only) && qa && tok_pos, "tqk_latent_absorb: null pointer");
     TQK_REQUIRE(n_heads > 0 && n_heads <= 65535 && dn > 0 && dr >= 0 && rk > 0 && n_tokens >= 0, "tqk_latent_absorb: bad sizes");
     TQK_REQUIRE(rot_dims >= 0 && rot_dims <= dr && rot_dims % 2 == 0, "tqk_latent_absorb: %d of %d elements rotate", rot_dims, dr);
     TQK_REQUIRE(rot_dims == 0 || (cos_table && sin_table && max_positions > 0), "tqk_latent_absorb: no angle tables");
@@ -275,7 +425,7 @@ extern "C" int tqk_latent_absorb(const void* q, int act_dtype, const void* w_uk,
     dim3 grid((n_tokens + LAT_TT - 1) / LAT_TT, n_heads);
 #define TQK_ABSORB(TA, TW)                                                                                                             \
     latent_absorb_kernel<TA, TW><<<grid, 128, lds, s>>>((const TA*)q, (const TW*)w_uk, n_heads, dn, dr, rk, cos_table, sin_table,      \
-                                                        rot_dims, max_positions, tok_pos, qa, n_tokens)
+                                                        rot_dims, max_positions, tok_pos, qa, n_tokens, tail_only)
     if (act_dtype == TQK_F32 && w_dtype == TQK_F32) TQK_ABSORB(float, float);
     else if (act_dtype == TQK_F32 && w_dtype == TQK_BF16) TQK_ABSORB(float, bf16_t);
     else if (act_dtype == TQK_BF16 && w_dtype == TQK_F32) TQK_ABSORB(bf16_t, float);
@@ -283,6 +433,33 @@ extern "C" int tqk_latent_absorb(const void* q, int act_dtype, const void* w_uk,
     else return tqk_fail("tqk_latent_absorb: unknown dtypes %d, %d", act_dtype, w_dtype);
 #undef TQK_ABSORB
     return tqk_check_launch("tqk_latent_absorb");
+}
+
+extern "C" int tqk_latent_attention_mfma_supported(int rk, int dr) { return (rk + dr) % 8 == 0 && rk <= LAT_MAX_RK && rk + dr <= LAT_MAX_DK; }
+
+extern "C" int tqk_latent_attention_mfma(const float* qa, const void* cache, const void* turned, const int32_t* tok_seq, const int32_t* tok_pos,
+                                         const int32_t* page_table, int table_width, int n_seqs, int n_pages, int window, float scale,
+                                         float* out, int n_tokens, int n_heads, int rk, int dr, void* stream) {
+    TQK_REQUIRE(qa && cache && turned && tok_seq && tok_pos && page_table && out, "tqk_latent_attention_mfma: null pointer");
+    TQK_REQUIRE(n_tokens >= 0 && n_heads > 0 && rk > 0 && dr >= 0, "tqk_latent_attention_mfma: bad sizes");
+    TQK_REQUIRE(tqk_latent_attention_mfma_supported(rk, dr), "tqk_latent_attention_mfma: a latent of %d + %d values is not taken", rk, dr);
+    TQK_REQUIRE(table_width > 0 && n_pages > 0 && n_seqs > 0 && window >= 0, "tqk_latent_attention_mfma: empty page table or negative window");
+    TQK_REQUIRE(((((uintptr_t)qa) | ((uintptr_t)cache) | ((uintptr_t)turned)) & 15) == 0, "tqk_latent_attention_mfma: operands must be 16-byte aligned");
+    if (n_tokens == 0) return 0;
+    const int dk = rk + dr, n_chunks = (n_heads + 15) / 16;
+    const long long items = (long long)n_tokens * n_chunks;
+    TQK_REQUIRE(items <= 0x7fffffffLL, "tqk_latent_attention_mfma: too many rows");
+    const unsigned blocks = (unsigned)((items + LAT_WAVES - 1) / LAT_WAVES);
+    hipStream_t s = (hipStream_t)stream;
+#define TQK_LAT_MFMA(KS, NCT)                                                                                                         \
+    latent_attention_mfma_kernel<KS, NCT><<<blocks, LAT_WAVES * TQK_WAVE, 0, s>>>(qa, (const bf16_t*)cache, (const bf16_t*)turned, tok_seq, \
+                                                                                  tok_pos, page_table, table_width, window, scale, out,   \
+                                                                                  n_tokens, n_heads, n_chunks, rk, dk)
+    if (rk <= 128 && dk <= 160) TQK_LAT_MFMA(5, 8);
+    else if (rk <= 256 && dk <= 320) TQK_LAT_MFMA(10, 16);
+    else TQK_LAT_MFMA(20, 32);
+#undef TQK_LAT_MFMA
+    return tqk_check_launch("tqk_latent_attention_mfma");
 }
 
 extern "C" int tqk_latent_attention(const float* qa, const void* cache, int cache_dtype, const int32_t* tok_seq, const int32_t* tok_pos,

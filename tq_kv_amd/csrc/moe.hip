@@ -22,35 +22,44 @@
 #define MOE_TK 16               // k per stage
 
 // ---- route -----------------------------------------------------------------------------------
+// A block per token: its waves share the experts out for the logits (each a dot product over the lanes, several loads
+// under way at once, added up in a fixed order), then the first wave takes the softmax and the largest.
 template <typename TA, typename TW>
 __global__ __launch_bounds__(MOE_ROUTE_WAVES * TQK_WAVE)
 void moe_route_kernel(const TA* __restrict__ x, const TW* __restrict__ w, int n_experts, int hidden, int top, float scale,
-                      int32_t* __restrict__ idx, float* __restrict__ weight, int n_tokens) {
-    __shared__ float z[MOE_ROUTE_WAVES][MOE_MAX_EXPERTS];
+                      int32_t* __restrict__ idx, float* __restrict__ weight) {
+    __shared__ float z[MOE_MAX_EXPERTS];
     const int wave = threadIdx.x / TQK_WAVE, lane = threadIdx.x % TQK_WAVE;
-    const int t_own = blockIdx.x * MOE_ROUTE_WAVES + wave;
-    const bool live = t_own < n_tokens;             // a wave without a token repeats the last one and writes nothing
-    const int t = live ? t_own : n_tokens - 1;
+    const int t = blockIdx.x;
     const TA* xr = x + (size_t)t * hidden;
-    for (int e = 0; e < n_experts; ++e) {
+    for (int e = wave; e < n_experts; e += MOE_ROUTE_WAVES) {
         const TW* wr = w + (size_t)e * hidden;
-        float dot = 0.f;
-        for (int i = lane; i < hidden; i += TQK_WAVE) dot = fmaf(to_float(xr[i]), to_float(wr[i]), dot);
-        dot = wave_sum(dot);
-        if (lane == 0) z[wave][e] = dot;
+        float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
+        int i = lane;
+        for (; i + 3 * TQK_WAVE < hidden; i += 4 * TQK_WAVE) {
+            d0 = fmaf(to_float(xr[i]), to_float(wr[i]), d0);
+            d1 = fmaf(to_float(xr[i + TQK_WAVE]), to_float(wr[i + TQK_WAVE]), d1);
+            d2 = fmaf(to_float(xr[i + 2 * TQK_WAVE]), to_float(wr[i + 2 * TQK_WAVE]), d2);
+            d3 = fmaf(to_float(xr[i + 3 * TQK_WAVE]), to_float(wr[i + 3 * TQK_WAVE]), d3);
+        }
+        for (; i < hidden; i += TQK_WAVE) d0 = fmaf(to_float(xr[i]), to_float(wr[i]), d0);
+        const float dot = wave_sum((d0 + d1) + (d2 + d3));
+        if (lane == 0) z[e] = dot;
     }
     __syncthreads();
+    if (wave != 0) return;
     float m = -INFINITY;
-    for (int e = lane; e < n_experts; e += TQK_WAVE) m = fmaxf(m, z[wave][e]);
+    for (int e = lane; e < n_experts; e += TQK_WAVE) m = fmaxf(m, z[e]);
     m = wave_max(m);
     float sum = 0.f;
-    for (int e = lane; e < n_experts; e += TQK_WAVE) sum += expf(z[wave][e] - m);
+    for (int e = lane; e < n_experts; e += TQK_WAVE) sum += expf(z[e] - m);
     sum = wave_sum(sum);
+    // what the lane's experts still offer; a chosen one is struck out in the registers of the lane that holds it
     for (int k = 0; k < top; ++k) {
         float best = -INFINITY;
         int best_e = 0x7fffffff;
         for (int e = lane; e < n_experts; e += TQK_WAVE) {
-            const float v = z[wave][e];
+            const float v = z[e];
             if (v > best) { best = v; best_e = e; }         // increasing e: the lower index stays on a tie
         }
 #pragma unroll
@@ -59,14 +68,11 @@ void moe_route_kernel(const TA* __restrict__ x, const TW* __restrict__ w, int n_
             const int oe = __shfl_xor(best_e, o, TQK_WAVE);
             if (ov > best || (ov == best && oe < best_e)) { best = ov; best_e = oe; }
         }
+        if (lane == best_e % TQK_WAVE) z[best_e] = -INFINITY;       // the lane that reads this expert writes it: no other sees it
         if (lane == 0) {
-            if (live) {
-                idx[(size_t)t * top + k] = best_e;
-                weight[(size_t)t * top + k] = expf(best - m) / sum * scale;
-            }
-            z[wave][best_e] = -INFINITY;
+            idx[(size_t)t * top + k] = best_e;
+            weight[(size_t)t * top + k] = expf(best - m) / sum * scale;
         }
-        __syncthreads();
     }
 }
 
@@ -198,7 +204,7 @@ void moe_combine_kernel(const TA* __restrict__ y, const int32_t* __restrict__ pa
 // ---- entry points ----------------------------------------------------------------------------
 extern "C" int tqk_moe_max_experts(void) { return MOE_MAX_EXPERTS; }
 extern "C" int tqk_moe_tile_rows(void) { return MOE_TM; }
-extern "C" int tqk_moe_max_tiles(int n_pairs, int n_experts) { return (n_pairs + MOE_TM - 1) / MOE_TM + n_experts; }
+extern "C" int tqk_moe_max_tiles(int n_pairs, int n_experts, int tile_m) { return (n_pairs + tile_m - 1) / tile_m + n_experts; }
 
 extern "C" int tqk_moe_route(const void* x, int act_dtype, const void* w_router, int w_dtype, int n_experts, int hidden, int top, float scale,
                              int32_t* idx, float* weight, int n_tokens, void* stream) {
@@ -207,9 +213,8 @@ extern "C" int tqk_moe_route(const void* x, int act_dtype, const void* w_router,
     TQK_REQUIRE(top > 0 && top <= n_experts && hidden > 0 && n_tokens >= 0, "tqk_moe_route: bad sizes (top %d of %d experts)", top, n_experts);
     if (n_tokens == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
-    const unsigned blocks = (unsigned)((n_tokens + MOE_ROUTE_WAVES - 1) / MOE_ROUTE_WAVES);
 #define TQK_ROUTE(TA, TW) \
-    moe_route_kernel<TA, TW><<<blocks, MOE_ROUTE_WAVES * TQK_WAVE, 0, s>>>((const TA*)x, (const TW*)w_router, n_experts, hidden, top, scale, idx, weight, n_tokens)
+    moe_route_kernel<TA, TW><<<n_tokens, MOE_ROUTE_WAVES * TQK_WAVE, 0, s>>>((const TA*)x, (const TW*)w_router, n_experts, hidden, top, scale, idx, weight)
     if (act_dtype == TQK_F32 && w_dtype == TQK_F32) TQK_ROUTE(float, float);
     else if (act_dtype == TQK_F32 && w_dtype == TQK_BF16) TQK_ROUTE(float, bf16_t);
     else if (act_dtype == TQK_BF16 && w_dtype == TQK_F32) TQK_ROUTE(bf16_t, float);
@@ -219,13 +224,14 @@ extern "C" int tqk_moe_route(const void* x, int act_dtype, const void* w_router,
     return tqk_check_launch("tqk_moe_route");
 }
 
-extern "C" int tqk_moe_group(const int32_t* idx, int n_tokens, int top, int n_experts, int32_t* pair_pos, int32_t* sorted_tok,
+extern "C" int tqk_moe_group(const int32_t* idx, int n_tokens, int top, int n_experts, int tile_m, int32_t* pair_pos, int32_t* sorted_tok,
                              int32_t* tile_expert, int32_t* tile_row0, int32_t* tile_rows, int32_t* n_tiles, void* stream) {
     TQK_REQUIRE(idx && pair_pos && sorted_tok && tile_expert && tile_row0 && tile_rows && n_tiles, "tqk_moe_group: null pointer");
     TQK_REQUIRE(n_experts > 0 && n_experts <= MOE_MAX_EXPERTS && top > 0 && n_tokens >= 0, "tqk_moe_group: bad sizes");
     TQK_REQUIRE((long long)n_tokens * top <= 0x7fffffff, "tqk_moe_group: too many pairs");
+    TQK_REQUIRE(tile_m > 0, "tqk_moe_group: tiles of %d rows", tile_m);
     if (n_tokens == 0) return 0;
-    moe_group_kernel<<<1, 1024, 0, (hipStream_t)stream>>>(idx, n_tokens * top, top, n_experts, MOE_TM, pair_pos, sorted_tok, tile_expert, tile_row0,
+    moe_group_kernel<<<1, 1024, 0, (hipStream_t)stream>>>(idx, n_tokens * top, top, n_experts, tile_m, pair_pos, sorted_tok, tile_expert, tile_row0,
                                                           tile_rows, n_tiles);
     return tqk_check_launch("tqk_moe_group");
 }
@@ -251,6 +257,7 @@ extern "C" int tqk_moe_product(const void* x, int act_dtype, const int32_t* x_ro
     TQK_REQUIRE(N > 0 && K > 0 && max_tiles >= 0 && max_tiles <= 65535, "tqk_moe_product: bad sizes (N %d, K %d, %d tiles)", N, K, max_tiles);
     TQK_REQUIRE(!gated || (gate >= 0 && gate < TQK_GATE_KINDS), "tqk_moe_product: unknown gate %d", gate);
     TQK_REQUIRE(expert_stride >= (long long)(gated ? 2 : 1) * N * K, "tqk_moe_product: experts overlap");
+    /* the tile lists must have been made for tiles of tqk_moe_tile_rows() rows */
     if (max_tiles == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
 #define TQK_MOE(TX, TW) \

@@ -190,23 +190,30 @@ int tqk_mid_gated_act(const void* x, const void* w_packed, void* y, int M, int N
  * tqk_latent_split: row t of proj (row_stride values) begins [q_rank | kv_rank + rot_dim (absent when kv_rank == 0) | n_gate].  cq_out
  * [tokens, q_rank] = RMS norm of the first part times q_norm_w; the second part goes into the cache row of the token's
  * position (RMS norm times kv_norm_w of its first kv_rank values, rotation in halves of the first rot_dims of the
- * others by the angle table row tok_pos[t]); gate_out [tokens, n_gate] = sigmoid of the last part, float32. */
+ * others by the angle table row tok_pos[t]; `turned`, if given, gets the latent a second time, pages [n_pages][kv_rank][64]
+ * with a page's positions at the places of the standard value pages, see tqk_rope_store); gate_out [tokens, n_gate] = sigmoid of the last part, float32. */
 int tqk_latent_max_rank(void);          /* the largest latent (rk) tqk_latent_attention takes */
 int tqk_latent_max_row(void);           /* the largest cache row (rk + dr) it takes */
 int tqk_latent_split(const void* proj, int act_dtype, int row_stride, int q_rank, int kv_rank, int rot_dim, int n_gate, const void* q_norm_w,
                      const void* kv_norm_w, int norm_dtype, float eps, const float* cos_table, const float* sin_table,
                      int rot_dims, int max_positions, const int32_t* tok_seq, const int32_t* tok_pos,
-                     const int32_t* page_table, int table_width, void* cache, int n_pages, void* cq_out, float* gate_out,
-                     int n_tokens, void* stream);
-/* qa [tokens, heads, rk + dr] float32: qa[:rk] = W_uk,h^T q[:dn] (w_uk [heads * dn, rk]), qa[rk:] = q[dn:] rotated */
+                     const int32_t* page_table, int table_width, void* cache, void* turned, int n_pages, void* cq_out,
+                     float* gate_out, int n_tokens, void* stream);
+/* qa [tokens, heads, rk + dr] float32: qa[:rk] = W_uk,h^T q[:dn] (w_uk [heads * dn, rk]), qa[rk:] = q[dn:] rotated;
+ * tail_only: the rotated part alone (the product is someone else's: tqk_head_product) */
 int tqk_latent_absorb(const void* q, int act_dtype, const void* w_uk, int w_dtype, int n_heads, int dn, int dr, int rk,
                       const float* cos_table, const float* sin_table, int rot_dims, int max_positions,
-                      const int32_t* tok_pos, float* qa, int n_tokens, void* stream);
+                      const int32_t* tok_pos, float* qa, int n_tokens, int tail_only, void* stream);
 /* out [tokens, heads, rk] float32 = softmax over the visible positions of (qa . row) * scale, times row[:rk];
  * visible: lo..tok_pos[t], lo = max(0, tok_pos - window + 1) if window > 0 else 0 */
 int tqk_latent_attention(const float* qa, const void* cache, int cache_dtype, const int32_t* tok_seq, const int32_t* tok_pos,
                          const int32_t* page_table, int table_width, int n_seqs, int n_pages, int window, float scale,
                          float* out, int n_tokens, int n_heads, int rk, int dr, void* stream);
+/* the same on the matrix cores, for a bfloat16 cache with its turned copy, where tqk_latent_attention_mfma_supported says so */
+int tqk_latent_attention_mfma_supported(int rk, int dr);
+int tqk_latent_attention_mfma(const float* qa, const void* cache, const void* turned, const int32_t* tok_seq, const int32_t* tok_pos,
+                              const int32_t* page_table, int table_width, int n_seqs, int n_pages, int window, float scale,
+                              float* out, int n_tokens, int n_heads, int rk, int dr, void* stream);
 /* y [tokens, heads * dv] = gate[t, h] * W_uv,h o[t, h] (w_uv [heads * dv, rk]; gate may be null) */
 int tqk_latent_values(const float* o, const void* w_uv, int w_dtype, const float* gate, int n_heads, int rk, int dv, void* y,
                       int y_dtype, int n_tokens, void* stream);
@@ -219,14 +226,25 @@ int tqk_latent_values(const float* o, const void* w_uv, int w_dtype, const float
  * y [pairs, N].  tqk_moe_combine: out[t] = sum_k weight[t, k] y[pair_pos[t, k]] + shared[t] (shared may be null). */
 int tqk_moe_max_experts(void);
 int tqk_moe_tile_rows(void);
-int tqk_moe_max_tiles(int n_pairs, int n_experts);
+int tqk_moe_max_tiles(int n_pairs, int n_experts, int tile_m);
 int tqk_moe_route(const void* x, int act_dtype, const void* w_router, int w_dtype, int n_experts, int hidden, int top, float scale,
                   int32_t* idx, float* weight, int n_tokens, void* stream);
-int tqk_moe_group(const int32_t* idx, int n_tokens, int top, int n_experts, int32_t* pair_pos, int32_t* sorted_tok,
+int tqk_moe_group(const int32_t* idx, int n_tokens, int top, int n_experts, int tile_m, int32_t* pair_pos, int32_t* sorted_tok,
                   int32_t* tile_expert, int32_t* tile_row0, int32_t* tile_rows, int32_t* n_tiles, void* stream);
 int tqk_moe_product(const void* x, int act_dtype, const int32_t* x_rows, const void* w, int w_dtype, long long expert_stride, void* y,
                     int N, int K, int gated, int gate, float limit, float alpha, const int32_t* tile_expert,
                     const int32_t* tile_row0, const int32_t* tile_rows, const int32_t* n_tiles, int max_tiles, void* stream);
+/* Many small products on the matrix cores (grouped.hip), bfloat16 weights, K a multiple of 8: the experts' products over
+ * tiles of up to tile_m rows (16, 32 or 64, what tqk_moe_group was given; tqk_moe_product takes tqk_moe_tile_rows()), and
+ * y[t, h, :N] = scale[t, h] * W_h x[t, h, :K] for every token and head (x bfloat16 or float32, w [heads][N][K], y
+ * bfloat16 or float32, strides in values, scale float32 [tokens, heads] or null). */
+int tqk_grouped_supported(int K);
+int tqk_moe_product_mfma(const void* x, const int32_t* x_rows, const void* w, long long expert_stride, void* y, int N, int K,
+                         int gated, int gate, float limit, float alpha, const int32_t* tile_expert, const int32_t* tile_row0,
+                         const int32_t* tile_rows, const int32_t* n_tiles, int max_tiles, int tile_m, void* stream);
+int tqk_head_product(const void* x, int x_f32, long long x_row_stride, long long x_head_stride, const void* w, void* y, int y_f32,
+                     long long y_row_stride, long long y_head_stride, const float* scale, int n_tokens, int n_heads, int N, int K,
+                     void* stream);
 int tqk_moe_combine(const void* y, int act_dtype, const int32_t* pair_pos, const float* weight, int top, const void* shared, void* out,
                     int n_tokens, int hidden, void* stream);
 

@@ -55,7 +55,8 @@ TQ_QUERY(int, latent_max_row);
 TQ_KERNEL(latent_split, cptr, int, int, int, int, int, int, cptr, cptr, int, float, cf32, cf32, int, int, ci32, ci32, ci32, int, void*, void*, int,
           void*, float*, int, void*);
 TQ_QUERY(int, latent_attention_mfma_supported, int, int);
-TQ_KERNEL(latent_attention_mfma, cf32, cptr, cptr, ci32, ci32, ci32, int, int, int, int, float, float*, int, int, int, int, void*);
+TQ_QUERY(int, latent_attention_parts, int, int, int, int);
+TQ_KERNEL(latent_attention_mfma, cf32, cptr, cptr, ci32, ci32, ci32, int, int, int, int, float, float*, int, int, int, int, int, float*, float*, void*);
 TQ_KERNEL(latent_absorb, cptr, int, cptr, int, int, int, int, int, cf32, cf32, int, int, ci32, float*, int, int, void*);
 TQ_KERNEL(latent_attention, cf32, cptr, int, ci32, ci32, ci32, int, int, int, int, float, float*, int, int, int, int, void*);
 TQ_KERNEL(latent_values, cf32, cptr, int, cf32, int, int, int, void*, int, int, void*);

@@ -185,10 +185,18 @@ public:
         K::latent_absorb(q.data, dtype, uk_->t.data, uk_->t.dtype, n_heads_, dn_, dr_, kv_rank_, cos, sin, rot_dims, max_pos, c.dev.tok_pos,
                          (float*)qa.data, (int)n, heads_on_cores ? 1 : 0, c.stream);
         Tensor o = c.alloc(F32, {n, n_heads_, kv_rank_});
-        if (on_cores)
+        if (on_cores) {
+            // few tokens (decoding): a token's pages go to several waves, whose results a second kernel merges
+            const int n_parts = K::latent_attention_parts.raw((int)n, n_heads_, table.width, window_);
+            Tensor part_o, part_ml;
+            if (n_parts > 1) {
+                part_o = c.alloc(F32, {n, n_heads_, n_parts, kv_rank_});
+                part_ml = c.alloc(F32, {n, n_heads_, n_parts, 2});
+            }
             K::latent_attention_mfma((const float*)qa.data, entry.keys.data, entry.values.data, c.dev.tok_seq, c.dev.tok_pos, table.dev, table.width,
-                                     c.n_seqs, n_pages, window_, scale_, (float*)o.data, (int)n, n_heads_, kv_rank_, dr_, c.stream);
-        else
+                                     c.n_seqs, n_pages, window_, scale_, (float*)o.data, (int)n, n_heads_, kv_rank_, dr_, n_parts,
+                                     (float*)part_o.data, (float*)part_ml.data, c.stream);
+        } else
             K::latent_attention((const float*)qa.data, entry.keys.data, entry.keys.dtype, c.dev.tok_seq, c.dev.tok_pos, table.dev, table.width, c.n_seqs,
                                 n_pages, window_, scale_, (float*)o.data, (int)n, n_heads_, kv_rank_, dr_, c.stream);
         Tensor y = c.alloc(dtype, {n, (int64_t)n_heads_ * dv_});

@@ -51,6 +51,10 @@ struct GroupedArgs {
 template <int RT, int CB, bool GATED>
 __global__ __launch_bounds__(GRP_WAVES * TQK_WAVE)
 void grouped_mfma_kernel(GroupedArgs p) {
+    // tiles of more than 16 rows: the block brings a step's rows of x into LDS once (one 16-byte piece a thread), in the
+    // order the lanes take them, two buffers in turn with one barrier a step; its waves read them from there
+    constexpr bool STAGE = RT > 1;
+    __shared__ uint4 x_lds[STAGE ? 2 : 1][4][STAGE ? 16 * RT : 1];
     int group, row0, n_rows;
     if (p.tile_group) {
         const int tile = blockIdx.y;
@@ -66,7 +70,8 @@ void grouped_mfma_kernel(GroupedArgs p) {
     const int wave = threadIdx.x / TQK_WAVE, lane = threadIdx.x % TQK_WAVE;
     const int g = lane / 16, r16 = lane % 16;
     const int n0 = (blockIdx.x * GRP_WAVES + wave) * CB * 16;
-    if (n0 >= p.N) return;
+    const bool active = n0 < p.N;
+    if (!STAGE && !active) return;
     constexpr int NB = GATED ? 2 : 1;
     grp_floatx4_t acc[NB][RT][CB];
 #pragma unroll
@@ -75,52 +80,85 @@ void grouped_mfma_kernel(GroupedArgs p) {
         for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb) acc[b][rt][cb] = grp_floatx4_t{0.f, 0.f, 0.f, 0.f};
-    // where the lane's rows of x and of the weight begin
+    // where the rows of x begin: the lane's own (no staging), or the one row whose pieces the thread stages
+    auto row_offset = [&](int r) -> long long {
+        return r < n_rows ? (long long)(p.x_rows ? p.x_rows[row0 + r] : row0 + r) * p.x_row_stride + (long long)group * p.x_group_stride : -1;
+    };
+    // (no branch on what is outside: such a lane reads a piece that exists and drops it, so that loads can be under way
+    // over several steps)
+    auto load_x = [&](long long off, int e0) -> uint4 {
+        grp_pack8 a;
+        const bool out = off < 0 || e0 + 8 > p.K;
+        if (off < 0) off = (long long)group * p.x_group_stride + (p.x_rows ? (long long)p.x_rows[row0] * p.x_row_stride : (long long)row0 * p.x_row_stride);
+        e0 = min(e0, p.K - 8);
+        if (p.x_f32) {
+            const float4* src = reinterpret_cast<const float4*>((const float*)p.x + off + e0);
+            const float4 lo = src[0], hi = src[1];
+            a.u[0] = float_to_bf16_bits(lo.x); a.u[1] = float_to_bf16_bits(lo.y);
+            a.u[2] = float_to_bf16_bits(lo.z); a.u[3] = float_to_bf16_bits(lo.w);
+            a.u[4] = float_to_bf16_bits(hi.x); a.u[5] = float_to_bf16_bits(hi.y);
+            a.u[6] = float_to_bf16_bits(hi.z); a.u[7] = float_to_bf16_bits(hi.w);
+        } else {
+            a.q = *reinterpret_cast<const uint4*>((const bf16_t*)p.x + off + e0);
+        }
+        if (out) a.q = make_uint4(0, 0, 0, 0);
+        return a.q;
+    };
     long long xoff[RT];
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
-        const int r = 16 * rt + r16;
-        xoff[rt] = r < n_rows ? (long long)(p.x_rows ? p.x_rows[row0 + r] : row0 + r) * p.x_row_stride + (long long)group * p.x_group_stride : -1;
-    }
+    for (int rt = 0; rt < RT; ++rt) xoff[rt] = STAGE ? -1 : row_offset(16 * rt + r16);
+    const int stage_row = threadIdx.x / 4, stage_g = threadIdx.x % 4;
+    const bool stages = STAGE && stage_row < 16 * RT;
+    const long long stage_off = stages ? row_offset(stage_row) : -1;
     const bf16_t* wg = p.w + (size_t)group * p.w_group_stride;
     long long woff[CB];
+    bool w_ok[CB];
 #pragma unroll
-    for (int cb = 0; cb < CB; ++cb) woff[cb] = n0 + 16 * cb + r16 < p.N ? (long long)(n0 + 16 * cb + r16) * p.K : -1;
+    for (int cb = 0; cb < CB; ++cb) {
+        w_ok[cb] = active && n0 + 16 * cb + r16 < p.N;
+        woff[cb] = (long long)(w_ok[cb] ? n0 + 16 * cb + r16 : 0) * p.K;
+    }
     const long long up = (long long)p.N * p.K;
 
-    for (int k0 = 0; k0 < p.K; k0 += 32) {
-        const int e0 = k0 + 8 * g;
-        const bool in = e0 + 8 <= p.K;
-        grp_pack8 a[RT], b[NB][CB];
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt) {
-            a[rt].q = make_uint4(0, 0, 0, 0);
-            if (in && xoff[rt] >= 0) {
-                if (p.x_f32) {
-                    const float4* src = reinterpret_cast<const float4*>((const float*)p.x + xoff[rt] + e0);
-                    const float4 lo = src[0], hi = src[1];
-                    a[rt].u[0] = float_to_bf16_bits(lo.x); a[rt].u[1] = float_to_bf16_bits(lo.y);
-                    a[rt].u[2] = float_to_bf16_bits(lo.z); a[rt].u[3] = float_to_bf16_bits(lo.w);
-                    a[rt].u[4] = float_to_bf16_bits(hi.x); a[rt].u[5] = float_to_bf16_bits(hi.y);
-                    a[rt].u[6] = float_to_bf16_bits(hi.z); a[rt].u[7] = float_to_bf16_bits(hi.w);
-                } else {
-                    a[rt].q = *reinterpret_cast<const uint4*>((const bf16_t*)p.x + xoff[rt] + e0);
-                }
-            }
-        }
+    // what the next step needs is asked for before this step's products: the weights' pieces and, where the rows of x are
+    // staged, the thread's piece of them
+    auto load_w = [&](int k0, grp_pack8 (&b)[NB][CB]) {
+        const int e0 = min(k0 + 8 * g, p.K - 8);
+        const bool in = k0 + 8 * g + 8 <= p.K;
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) {
-            const bool w_in = in && woff[cb] >= 0;
+            const bool w_in = in && w_ok[cb];
             // tiles of up to 16 rows read a weight once: such loads say so
             const grp_bf16x8_t* w0 = reinterpret_cast<const grp_bf16x8_t*>(wg + woff[cb] + e0);
             const grp_bf16x8_t* w1 = reinterpret_cast<const grp_bf16x8_t*>(wg + up + woff[cb] + e0);
-            b[0][cb].q = make_uint4(0, 0, 0, 0);
-            if (w_in) b[0][cb].v = RT == 1 ? __builtin_nontemporal_load(w0) : *w0;
+            b[0][cb].v = RT == 1 ? __builtin_nontemporal_load(w0) : *w0;
+            if (!w_in) b[0][cb].q = make_uint4(0, 0, 0, 0);
             if (GATED) {
-                b[NB - 1][cb].q = make_uint4(0, 0, 0, 0);
-                if (w_in) b[NB - 1][cb].v = RT == 1 ? __builtin_nontemporal_load(w1) : *w1;
+                b[NB - 1][cb].v = RT == 1 ? __builtin_nontemporal_load(w1) : *w1;
+                if (!w_in) b[NB - 1][cb].q = make_uint4(0, 0, 0, 0);
             }
         }
+    };
+    grp_pack8 b_next[NB][CB];
+    uint4 x_next = make_uint4(0, 0, 0, 0);
+    load_w(0, b_next);
+    if (stages) x_next = load_x(stage_off, 8 * stage_g);
+    for (int k0 = 0, step = 0; k0 < p.K; k0 += 32, ++step) {
+        grp_pack8 a[RT], b[NB][CB];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) b[nb][cb] = b_next[nb][cb];
+        if (STAGE) {
+            if (stages) x_lds[step & 1][stage_g][stage_row] = x_next;
+            __syncthreads();
+        }
+        if (k0 + 32 < p.K) {
+            load_w(k0 + 32, b_next);
+            if (stages) x_next = load_x(stage_off, k0 + 32 + 8 * stage_g);
+        }
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) a[rt].q = STAGE ? x_lds[step & 1][g][STAGE ? 16 * rt + r16 : 0] : load_x(xoff[rt], k0 + 8 * g);
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
@@ -129,6 +167,7 @@ void grouped_mfma_kernel(GroupedArgs p) {
                 for (int cb = 0; cb < CB; ++cb)
                     acc[nb][rt][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[rt].v, b[nb][cb].v, acc[nb][rt][cb], 0, 0, 0);
     }
+    if (!active) return;
     // the lane holds, of each block, feature n0 + 16 cb + r16 of rows 16 rt + 4 g + i
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt)
@@ -159,12 +198,14 @@ void grouped_mfma_kernel(GroupedArgs p) {
 template <bool GATED>
 static int launch_grouped(const GroupedArgs& a, int tiles, hipStream_t s) {
     // rows of a tile: up to 16, 32 or 64; features of a wave: 16 or 32 (32 where there are enough of them to fill the chip)
+    // tiles of more than 16 rows share their rows of x through LDS and keep 32 (gated) or 64 features a wave, so that what is
+    // loaded serves many products; tiles of up to 16 rows stream the weights, 16 features a wave, 32 where there are many
     const int rt = a.tile_rows_max > 32 ? 4 : a.tile_rows_max > 16 ? 2 : 1;
-    const int cb = ((long long)a.N / 16) * tiles >= 4096 && !GATED ? 2 : 1;
+    const int cb = rt > 1 ? (GATED ? 2 : (a.N >= 256 ? 4 : 2)) : (((long long)a.N / 16) * tiles >= 4096 && !GATED ? 2 : 1);
     dim3 grid((a.N + GRP_WAVES * cb * 16 - 1) / (GRP_WAVES * cb * 16), tiles);
 #define TQK_GRP(RT, CB) grouped_mfma_kernel<RT, CB, GATED><<<grid, GRP_WAVES * TQK_WAVE, 0, s>>>(a)
-    if (rt == 4) { if (cb == 2) TQK_GRP(4, 2); else TQK_GRP(4, 1); }
-    else if (rt == 2) { if (cb == 2) TQK_GRP(2, 2); else TQK_GRP(2, 1); }
+    if (rt == 4) { if (cb == 4) TQK_GRP(4, 4); else TQK_GRP(4, 2); }
+    else if (rt == 2) { if (cb == 4) TQK_GRP(2, 4); else TQK_GRP(2, 2); }
     else { if (cb == 2) TQK_GRP(1, 2); else TQK_GRP(1, 1); }
 #undef TQK_GRP
     return tqk_check_launch("tqk grouped product");

@@ -16,6 +16,8 @@
 // Norms, angles, scores, softmax weights, gates and all sums are float32; qa and o stay float32
 // between the kernels.  The order of a query's operations depends on its position alone.
 // Cache pages: [position in page][rk + dr].
+#include <algorithm>
+
 #include "common.h"
 #include "tq_kernels.h"
 
@@ -212,59 +214,71 @@ union lat_pack8 {
     uint4 q;
 };
 
-template <int KS, int NCT>
-__global__ __launch_bounds__(LAT_WAVES * TQK_WAVE)
+// WAVES: waves of a block (each with a token's 16 heads of its own; the queries wait in LDS, 1 KB per step and wave).
+// n_parts > 1: a token's pages are dealt out to that many waves, which leave their sums, maxima and weights for
+// latent_merge_kernel (decoding steps, where the tokens alone are too few waves).
+template <int KS, int NCT, int WAVES>
+__global__ __launch_bounds__(WAVES * TQK_WAVE)
 void latent_attention_mfma_kernel(const float* __restrict__ qa, const bf16_t* __restrict__ cache, const bf16_t* __restrict__ turned,
                                   const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos,
                                   const int32_t* __restrict__ page_table, int table_width, int window, float scale,
-                                  float* __restrict__ out, int n_tokens, int n_heads, int n_chunks, int rk, int dk) {
+                                  float* __restrict__ out, int n_tokens, int n_heads, int n_chunks, int rk, int dk, int n_parts,
+                                  float* __restrict__ part_o, float* __restrict__ part_ml) {
+    __shared__ uint4 q_lds[WAVES][KS][TQK_WAVE];
     const int wave = threadIdx.x / TQK_WAVE, lane = threadIdx.x % TQK_WAVE;
-    const int item = blockIdx.x * LAT_WAVES + wave;
-    if (item >= n_tokens * n_chunks) return;
-    const int t = item / n_chunks, head = (item % n_chunks) * 16 + lane % 16;
+    const int item = blockIdx.x * WAVES + wave;
+    if (item >= n_tokens * n_chunks * n_parts) return;
+    const int part = item % n_parts;
+    const int t = (item / n_parts) / n_chunks, head = ((item / n_parts) % n_chunks) * 16 + lane % 16;
     const int g = lane / 16, r16 = lane % 16;
     const int pos = tok_pos[t];
     const int32_t* pages = page_table + (size_t)tok_seq[t] * table_width;
     const int lo = window > 0 ? max(0, pos - window + 1) : 0;
     const int ks_used = (dk + 31) / 32, ct_used = (rk + 15) / 16;
+    (void)ct_used;
 
-    lat_pack8 bq[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
         const int e0 = 32 * ks + 8 * g;
-        bq[ks].q = make_uint4(0, 0, 0, 0);
-        if (head < n_heads && e0 + 8 <= dk) {
+        lat_pack8 bq;
+        bq.q = make_uint4(0, 0, 0, 0);
+        if (ks < ks_used && head < n_heads && e0 + 8 <= dk) {
             const float4* src = reinterpret_cast<const float4*>(qa + ((size_t)t * n_heads + head) * dk + e0);
             const float4 a = src[0], b = src[1];
-            bq[ks].u[0] = float_to_bf16_bits(a.x); bq[ks].u[1] = float_to_bf16_bits(a.y);
-            bq[ks].u[2] = float_to_bf16_bits(a.z); bq[ks].u[3] = float_to_bf16_bits(a.w);
-            bq[ks].u[4] = float_to_bf16_bits(b.x); bq[ks].u[5] = float_to_bf16_bits(b.y);
-            bq[ks].u[6] = float_to_bf16_bits(b.z); bq[ks].u[7] = float_to_bf16_bits(b.w);
+            bq.u[0] = float_to_bf16_bits(a.x); bq.u[1] = float_to_bf16_bits(a.y);
+            bq.u[2] = float_to_bf16_bits(a.z); bq.u[3] = float_to_bf16_bits(a.w);
+            bq.u[4] = float_to_bf16_bits(b.x); bq.u[5] = float_to_bf16_bits(b.y);
+            bq.u[6] = float_to_bf16_bits(b.z); bq.u[7] = float_to_bf16_bits(b.w);
         }
+        q_lds[wave][ks][lane] = bq.q;           // read back by the lane that wrote it: no barrier
     }
     lat_floatx4_t o[NCT];
 #pragma unroll
     for (int ct = 0; ct < NCT; ++ct) o[ct] = lat_floatx4_t{0.f, 0.f, 0.f, 0.f};
     float m = -INFINITY, l = 0.f;
 
-    for (int kb = (lo / TQK_PAGE) * TQK_PAGE; kb <= pos; kb += TQK_PAGE) {
+    for (int kb = (lo / TQK_PAGE + part) * TQK_PAGE; kb <= pos; kb += TQK_PAGE * n_parts) {
         const int page = max(0, pages[kb / TQK_PAGE]);
         const bf16_t* kp = cache + (size_t)page * TQK_PAGE * dk;
         const bf16_t* vp = turned + (size_t)page * rk * TQK_PAGE;
         lat_floatx4_t s[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) s[j] = lat_floatx4_t{0.f, 0.f, 0.f, 0.f};
+        // (no branch inside: a lane whose piece lies beyond the row reads the row's last piece instead and drops it, so
+        // that the loads of many steps can be under way at once)
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            if (ks < ks_used) {
-                const int e0 = 32 * ks + 8 * g;
-                const bool in = e0 + 8 <= dk;
+            const int e0 = 32 * ks + 8 * g;
+            const bool in = e0 + 8 <= dk;
+            const int e0c = in ? e0 : dk - 8;
+            lat_pack8 bq;
+            bq.q = q_lds[wave][ks][lane];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    lat_pack8 a;
-                    a.q = in ? *reinterpret_cast<const uint4*>(kp + (size_t)(16 * j + r16) * dk + e0) : make_uint4(0, 0, 0, 0);
-                    s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, bq[ks].v, s[j], 0, 0, 0);
-                }
+            for (int j = 0; j < 4; ++j) {
+                lat_pack8 a;
+                a.q = *reinterpret_cast<const uint4*>(kp + (size_t)(16 * j + r16) * dk + e0c);
+                if (!in) a.q = make_uint4(0, 0, 0, 0);
+                s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, bq.v, s[j], 0, 0, 0);
             }
         }
         // the lane's 16 scores belong to its head and keys kb + 16 j + 4 g + i
@@ -304,28 +318,28 @@ void latent_attention_mfma_kernel(const float* __restrict__ qa, const bf16_t* __
         const bool edge = kb < lo || kb + TQK_PAGE - 1 > pos;
 #pragma unroll
         for (int ct = 0; ct < NCT; ++ct) {
-            if (ct < ct_used) {
-                const int col = 16 * ct + r16;
-                o[ct] *= alpha;
+            const int col = 16 * ct + r16;
+            const int colc = min(col, rk - 1);
+            o[ct] *= alpha;
 #pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    lat_pack8 a;
-                    a.q = col < rk ? *reinterpret_cast<const uint4*>(vp + (size_t)col * TQK_PAGE + 32 * h + 8 * g) : make_uint4(0, 0, 0, 0);
-                    if (edge) {
+            for (int h = 0; h < 2; ++h) {
+                lat_pack8 a;
+                a.q = *reinterpret_cast<const uint4*>(vp + (size_t)colc * TQK_PAGE + 32 * h + 8 * g);
+                if (col >= rk) a.q = make_uint4(0, 0, 0, 0);
+                if (edge) {
 #pragma unroll
-                        for (int e = 0; e < 8; ++e) {
-                            const int key = kb + value_position(32 * h + 8 * g + e);
-                            if (key < lo || key > pos) a.u[e] = 0;
-                        }
+                    for (int e = 0; e < 8; ++e) {
+                        const int key = kb + value_position(32 * h + 8 * g + e);
+                        if (key < lo || key > pos) a.u[e] = 0;
                     }
-                    o[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pb[h].v, o[ct], 0, 0, 0);
                 }
+                o[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pb[h].v, o[ct], 0, 0, 0);
             }
         }
     }
     if (head >= n_heads) return;
-    float* dst = out + ((size_t)t * n_heads + head) * rk;
-    const float inv = 1.f / l;
+    float* dst = n_parts > 1 ? part_o + (((size_t)t * n_heads + head) * n_parts + part) * rk : out + ((size_t)t * n_heads + head) * rk;
+    const float inv = n_parts > 1 ? 1.f : 1.f / l;
 #pragma unroll
     for (int ct = 0; ct < NCT; ++ct) {
         if (ct < ct_used) {
@@ -335,6 +349,30 @@ void latent_attention_mfma_kernel(const float* __restrict__ qa, const bf16_t* __
                 if (col < rk) dst[col] = o[ct][i] * inv;
             }
         }
+    }
+    if (n_parts > 1 && g == 0) {
+        float* ml = part_ml + (((size_t)t * n_heads + head) * n_parts + part) * 2;
+        ml[0] = m;                  // -inf and 0 where the part had no page
+        ml[1] = l;
+    }
+}
+
+// the parts of a (token, head) in their order: out = sum_p o_p e^(m_p - M) / sum_p l_p e^(m_p - M)
+__global__ __launch_bounds__(128)
+void latent_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml, int n_parts, int rk, float* __restrict__ out) {
+    const size_t row = blockIdx.x;
+    const float* ml = part_ml + row * n_parts * 2;
+    float M = -INFINITY;
+    for (int p = 0; p < n_parts; ++p) M = fmaxf(M, ml[2 * p]);
+    float L = 0.f;
+    for (int p = 0; p < n_parts; ++p) L += ml[2 * p + 1] * expf(ml[2 * p] - M);
+    for (int c = threadIdx.x; c < rk; c += blockDim.x) {
+        float v = 0.f;
+        for (int p = 0; p < n_parts; ++p) {
+            const float wgt = expf(ml[2 * p] - M);
+            if (wgt > 0.f) v = fmaf(part_o[(row * n_parts + p) * rk + c], wgt, v);
+        }
+        out[row * rk + c] = v / L;
     }
 }
 
@@ -437,9 +475,19 @@ extern "C" int tqk_latent_absorb(const void* q, int act_dtype, const void* w_uk,
 
 extern "C" int tqk_latent_attention_mfma_supported(int rk, int dr) { return (rk + dr) % 8 == 0 && rk <= LAT_MAX_RK && rk + dr <= LAT_MAX_DK; }
 
+/* how many waves a token's pages are best dealt out to (1: none of it), and the scratch memory that takes */
+extern "C" int tqk_latent_attention_parts(int n_tokens, int n_heads, int table_width, int window) {
+    const long long items = (long long)n_tokens * ((n_heads + 15) / 16);
+    const int pages = window > 0 ? std::min(table_width, (window + TQK_PAGE - 2) / TQK_PAGE + 1) : table_width;
+    if (items >= 512 || pages <= 1) return 1;
+    return (int)std::max(1LL, std::min((long long)pages, 1024 / std::max(1LL, items)));
+}
+
 extern "C" int tqk_latent_attention_mfma(const float* qa, const void* cache, const void* turned, const int32_t* tok_seq, const int32_t* tok_pos,
                                          const int32_t* page_table, int table_width, int n_seqs, int n_pages, int window, float scale,
-                                         float* out, int n_tokens, int n_heads, int rk, int dr, void* stream) {
+                                         float* out, int n_tokens, int n_heads, int rk, int dr, int n_parts, float* part_o, float* part_ml,
+                                         void* stream) {
+    TQK_REQUIRE(n_parts >= 1 && (n_parts == 1 || (part_o && part_ml)), "tqk_latent_attention_mfma: %d parts without memory for them", n_parts);
     TQK_REQUIRE(qa && cache && turned && tok_seq && tok_pos && page_table && out, "tqk_latent_attention_mfma: null pointer");
     TQK_REQUIRE(n_tokens >= 0 && n_heads > 0 && rk > 0 && dr >= 0, "tqk_latent_attention_mfma: bad sizes");
     TQK_REQUIRE(tqk_latent_attention_mfma_supported(rk, dr), "tqk_latent_attention_mfma: a latent of %d + %d values is not taken", rk, dr);
@@ -447,19 +495,25 @@ extern "C" int tqk_latent_attention_mfma(const float* qa, const void* cache, con
     TQK_REQUIRE(((((uintptr_t)qa) | ((uintptr_t)cache) | ((uintptr_t)turned)) & 15) == 0, "tqk_latent_attention_mfma: operands must be 16-byte aligned");
     if (n_tokens == 0) return 0;
     const int dk = rk + dr, n_chunks = (n_heads + 15) / 16;
-    const long long items = (long long)n_tokens * n_chunks;
+    const long long items = (long long)n_tokens * n_chunks * n_parts;
     TQK_REQUIRE(items <= 0x7fffffffLL, "tqk_latent_attention_mfma: too many rows");
-    const unsigned blocks = (unsigned)((items + LAT_WAVES - 1) / LAT_WAVES);
     hipStream_t s = (hipStream_t)stream;
-#define TQK_LAT_MFMA(KS, NCT)                                                                                                         \
-    latent_attention_mfma_kernel<KS, NCT><<<blocks, LAT_WAVES * TQK_WAVE, 0, s>>>(qa, (const bf16_t*)cache, (const bf16_t*)turned, tok_seq, \
-                                                                                  tok_pos, page_table, table_width, window, scale, out,   \
-                                                                                  n_tokens, n_heads, n_chunks, rk, dk)
-    if (rk <= 128 && dk <= 160) TQK_LAT_MFMA(5, 8);
-    else if (rk <= 256 && dk <= 320) TQK_LAT_MFMA(10, 16);
-    else TQK_LAT_MFMA(20, 32);
+#define TQK_LAT_MFMA(KS, NCT, WAVES)                                                                                                  \
+    latent_attention_mfma_kernel<KS, NCT, WAVES><<<(unsigned)((items + WAVES - 1) / WAVES), WAVES * TQK_WAVE, 0, s>>>(                  \
+        qa, (const bf16_t*)cache, (const bf16_t*)turned, tok_seq, tok_pos, page_table, table_width, window, scale, out, n_tokens, n_heads, \
+        n_chunks, rk, dk, n_parts, part_o, part_ml)
+    // the smallest build that holds the row and the latent (steps and blocks beyond the sizes multiply zeros)
+    if (rk <= 128 && dk <= 160) TQK_LAT_MFMA(5, 8, 4);
+    else if (rk <= 256 && dk <= 320) TQK_LAT_MFMA(10, 16, 4);
+    else if (dk <= 576) TQK_LAT_MFMA(18, 32, 2);
+    else TQK_LAT_MFMA(20, 32, 2);
 #undef TQK_LAT_MFMA
-    return tqk_check_launch("tqk_latent_attention_mfma");
+    if (tqk_check_launch("tqk_latent_attention_mfma")) return -1;
+    if (n_parts > 1) {
+        latent_merge_kernel<<<(unsigned)(n_tokens * n_heads), 128, 0, s>>>(part_o, part_ml, n_parts, rk, out);
+        return tqk_check_launch("tqk_latent_attention_mfma merge");
+    }
+    return 0;
 }
 
 extern "C" int tqk_latent_attention(const float* qa, const void* cache, int cache_dtype, const int32_t* tok_seq, const int32_t* tok_pos,

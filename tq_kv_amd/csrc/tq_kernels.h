@@ -211,9 +211,13 @@ int tqk_latent_attention(const float* qa, const void* cache, int cache_dtype, co
                          float* out, int n_tokens, int n_heads, int rk, int dr, void* stream);
 /* the same on the matrix cores, for a bfloat16 cache with its turned copy, where tqk_latent_attention_mfma_supported says so */
 int tqk_latent_attention_mfma_supported(int rk, int dr);
+/* n_parts > 1: a token's pages are dealt out to that many waves and merged by a second kernel; part_o float32 [tokens,
+ * heads, n_parts, rk] and part_ml [tokens, heads, n_parts, 2] are its scratch.  tqk_latent_attention_parts: a good number. */
+int tqk_latent_attention_parts(int n_tokens, int n_heads, int table_width, int window);
 int tqk_latent_attention_mfma(const float* qa, const void* cache, const void* turned, const int32_t* tok_seq, const int32_t* tok_pos,
                               const int32_t* page_table, int table_width, int n_seqs, int n_pages, int window, float scale,
-                              float* out, int n_tokens, int n_heads, int rk, int dr, void* stream);
+                              float* out, int n_tokens, int n_heads, int rk, int dr, int n_parts, float* part_o, float* part_ml,
+                              void* stream);
 /* y [tokens, heads * dv] = gate[t, h] * W_uv,h o[t, h] (w_uv [heads * dv, rk]; gate may be null) */
 int tqk_latent_values(const float* o, const void* w_uv, int w_dtype, const float* gate, int n_heads, int rk, int dv, void* y,
                       int y_dtype, int n_tokens, void* stream);

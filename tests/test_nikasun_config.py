@@ -18,7 +18,8 @@ def test_the_architecture_is_known_by_its_name():
     assert "Nikasun" in known_architectures()
     name, typed = config_from_dict(N.config_mixed())
     assert name == "Nikasun"
-    typed = typed if isinstance(typed, dict) else typed.to_typed()
+    assert config_from_dict(typed.to_dict())[1] == typed and typed.layers[3].mixer.kv_from == 0          # round trip through config.json
+    typed = typed.to_typed()
     assert (typed["vocab"], typed["width"], typed["norm_eps"], typed["embedding_scale"]) == (331, 96, 3e-6, 7.5)
     assert [l["mixer"]["kv_from"] for l in typed["layers"]] == [None, None, None, 0, 2]
     assert [None if l["mlp"] is None else l["mlp"]["kind"] for l in typed["layers"]] == ["moe", None, "dense", "moe", "dense"]

@@ -50,7 +50,7 @@ def _add_model(p):
 
 
 def build_parser():
-    ap = argparse.ArgumentParser(prog="tq", description="tq for MI355X -- local LLM inference (Qwen2 dense decoder)")
+    ap = argparse.ArgumentParser(prog="tq", description="tq for MI355X -- local LLM inference (Qwen2 dense decoder, Nikasun latent-attention decoder)")
     ap.add_argument("--fp32", action="store_true", help="Run everything in true 32-bit (same as --dtype float32)")
     ap.add_argument("--trace", action="store_true",
                     help="Named ranges (model, attn, attn-mlp, rms-norm, output) around the parts of every step, for a profiler's marker trace")
@@ -202,6 +202,11 @@ def cmd_list(args):
     from .config import catalog
     for name, tag in catalog.entries():
         raw = catalog.find("%s:%s" % (name, tag))
+        if "num_hidden_layers" not in raw:          # an architecture that lists its layers one by one
+            kinds = ["none" if l.get("mlp") is None else l["mlp"]["kind"] for l in raw["layers"]]
+            print("%-16s %s layers=%-3d hidden=%-5d feed-forwards=%s vocab=%d"
+                  % ("%s:%s" % (name, tag), raw.get("architecture", "?"), len(raw["layers"]), raw["width"], ",".join(kinds), raw["vocab"]))
+            continue
         print("%-16s layers=%-3d hidden=%-5d heads=%d/%d head_dim=%d inter=%d vocab=%d"
               % ("%s:%s" % (name, tag), raw["num_hidden_layers"], raw["hidden_size"], raw["num_attention_heads"],
                  raw.get("num_key_value_heads", raw["num_attention_heads"]),

@@ -142,7 +142,8 @@ void grouped_mfma_kernel(GroupedArgs p) {
     grp_pack8 b_next[NB][CB];
     uint4 x_next = make_uint4(0, 0, 0, 0);
     load_w(0, b_next);
-    if (stages) x_next = load_x(stage_off, 8 * stage_g);
+    if (STAGE) x_next = load_x(stage_off, 8 * stage_g);
+    const int k_last = ((p.K - 1) / 32) * 32;
     for (int k0 = 0, step = 0; k0 < p.K; k0 += 32, ++step) {
         grp_pack8 a[RT], b[NB][CB];
 #pragma unroll
@@ -153,10 +154,9 @@ void grouped_mfma_kernel(GroupedArgs p) {
             if (stages) x_lds[step & 1][stage_g][stage_row] = x_next;
             __syncthreads();
         }
-        if (k0 + 32 < p.K) {
-            load_w(k0 + 32, b_next);
-            if (stages) x_next = load_x(stage_off, k0 + 32 + 8 * stage_g);
-        }
+        // (after the last step this asks for the last step's again and drops it: no branch between the loads)
+        load_w(min(k0 + 32, k_last), b_next);
+        if (STAGE) x_next = load_x(stage_off, min(k0 + 32, k_last) + 8 * stage_g);
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) a[rt].q = STAGE ? x_lds[step & 1][g][STAGE ? 16 * rt + r16 : 0] : load_x(xoff[rt], k0 + 8 * g);
 #pragma unroll

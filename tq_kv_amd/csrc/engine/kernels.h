@@ -56,6 +56,7 @@ TQ_KERNEL(latent_split, cptr, int, int, int, int, int, int, cptr, cptr, int, flo
           void*, float*, int, void*);
 TQ_QUERY(int, latent_attention_mfma_supported, int, int);
 TQ_QUERY(int, latent_attention_parts, int, int, int, int);
+TQ_KERNEL(latent_attention_tiles, cf32, cptr, cptr, ci32, ci32, int, int, int, ci32, ci32, ci32, int, int, float, float*, int, int, int, int, void*);
 TQ_KERNEL(latent_attention_mfma, cf32, cptr, cptr, ci32, ci32, ci32, int, int, int, int, float, float*, int, int, int, int, int, float*, float*, void*);
 TQ_KERNEL(latent_absorb, cptr, int, cptr, int, int, int, int, int, cf32, cf32, int, int, ci32, float*, int, int, void*);
 TQ_KERNEL(latent_attention, cf32, cptr, int, ci32, ci32, ci32, int, int, int, int, float, float*, int, int, int, int, void*);

@@ -185,7 +185,13 @@ public:
         K::latent_absorb(q.data, dtype, uk_->t.data, uk_->t.dtype, n_heads_, dn_, dr_, kv_rank_, cos, sin, rot_dims, max_pos, c.dev.tok_pos,
                          (float*)qa.data, (int)n, heads_on_cores ? 1 : 0, c.stream);
         Tensor o = c.alloc(F32, {n, n_heads_, kv_rank_});
-        if (on_cores) {
+        if (on_cores && !c.all_decode && !c.capturing) {
+            // several tokens per sequence: tiles of four consecutive tokens share what they read of the cache
+            const Tiles tl = c.query_tiles(4);
+            K::latent_attention_tiles((const float*)qa.data, entry.keys.data, entry.values.data, c.dev.tok_pos, table.dev, table.width, c.n_seqs,
+                                      n_pages, tl.seq, tl.tok0, tl.count, tl.n, window_, scale_, (float*)o.data, (int)n, n_heads_, kv_rank_, dr_,
+                                      c.stream);
+        } else if (on_cores) {
             // few tokens (decoding): a token's pages go to several waves, whose results a second kernel merges
             const int n_parts = K::latent_attention_parts.raw((int)n, n_heads_, table.width, window_);
             Tensor part_o, part_ml;

@@ -376,6 +376,185 @@ void latent_merge_kernel(const float* __restrict__ part_o, const float* __restri
     }
 }
 
+// ---- attention on the matrix cores, tiles of queries (prompts) -----------------------------------
+// A block of four waves takes up to four consecutive tokens of one sequence, a wave a token's 16 heads.  The products
+// are those of the kernel above; what differs is where the cache comes from: the block brings half a page (32
+// positions) of rows, then of turned latents, into LDS in the order the lanes take them, once for all four tokens, so
+// the cache is read a quarter as often.  A thread's pieces of the next half are asked for before the products on
+// this one and written to LDS after the barrier that ends them (rows while the second product runs, turned latents
+// while the first does).  The absorbed queries stay in registers.
+template <int KS, int NCT>
+__global__ __launch_bounds__(4 * TQK_WAVE)
+void latent_attention_tile_kernel(const float* __restrict__ qa, const bf16_t* __restrict__ cache, const bf16_t* __restrict__ turned,
+                                  const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ page_table, int table_width,
+                                  const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_tok0,
+                                  const int32_t* __restrict__ tile_count, int window, float scale, float* __restrict__ out, int n_heads,
+                                  int rk, int dk) {
+    constexpr int SLOTS = (2 * KS > NCT ? 2 * KS : NCT) * TQK_WAVE;
+    constexpr int KP = (128 * KS + 255) / 256;          // 16-byte pieces of half a page of rows a thread brings
+    constexpr int VP = NCT / 4;                         // and of turned latents
+    __shared__ uint4 lds[SLOTS];
+    const int tile = blockIdx.x;
+    const int tok0 = tile_tok0[tile], count = min(4, tile_count[tile]);
+    const int32_t* pages = page_table + (size_t)tile_seq[tile] * table_width;
+    const int wave = threadIdx.x / TQK_WAVE, lane = threadIdx.x % TQK_WAVE;
+    const int g = lane / 16, r16 = lane % 16;
+    const bool has = wave < count;
+    const int t = tok0 + min(wave, count - 1);
+    const int head = blockIdx.y * 16 + r16;
+    const int pos = tok_pos[t];
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int pos_max = tok_pos[tok0 + count - 1];
+    const int lo_min = window > 0 ? max(0, tok_pos[tok0] - window + 1) : 0;
+
+    lat_pack8 bq[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        const int e0 = 32 * ks + 8 * g;
+        bq[ks].q = make_uint4(0, 0, 0, 0);
+        if (has && head < n_heads && e0 + 8 <= dk) {
+            const float4* src = reinterpret_cast<const float4*>(qa + ((size_t)t * n_heads + head) * dk + e0);
+            const float4 a = src[0], b = src[1];
+            bq[ks].u[0] = float_to_bf16_bits(a.x); bq[ks].u[1] = float_to_bf16_bits(a.y);
+            bq[ks].u[2] = float_to_bf16_bits(a.z); bq[ks].u[3] = float_to_bf16_bits(a.w);
+            bq[ks].u[4] = float_to_bf16_bits(b.x); bq[ks].u[5] = float_to_bf16_bits(b.y);
+            bq[ks].u[6] = float_to_bf16_bits(b.z); bq[ks].u[7] = float_to_bf16_bits(b.w);
+        }
+    }
+    lat_floatx4_t o[NCT];
+#pragma unroll
+    for (int ct = 0; ct < NCT; ++ct) o[ct] = lat_floatx4_t{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+
+    // a thread's pieces of half a page: rows (piece i: position i / (4 KS) of the half, elements 8 (i % (4 KS)) on)
+    uint4 k_regs[KP], v_regs[VP];
+    auto fetch_rows = [&](int hp) {
+        const int page = max(0, pages[hp / 2]);
+        const bf16_t* kp = cache + ((size_t)page * TQK_PAGE + (size_t)(hp & 1) * 32) * dk;
+#pragma unroll
+        for (int n = 0; n < KP; ++n) {
+            const int i = threadIdx.x + n * 256;
+            const int key = min(i / (4 * KS), 31), e = i % (4 * KS);
+            const bool in = 8 * e + 8 <= dk;
+            k_regs[n] = *reinterpret_cast<const uint4*>(kp + (size_t)key * dk + (in ? 8 * e : 0));
+            if (!in) k_regs[n] = make_uint4(0, 0, 0, 0);
+        }
+    };
+    auto store_rows = [&]() {
+#pragma unroll
+        for (int n = 0; n < KP; ++n) {
+            const int i = threadIdx.x + n * 256;
+            if (i >= 128 * KS) continue;
+            const int key = i / (4 * KS), e = i % (4 * KS);
+            lds[((key / 16) * KS + e / 4) * TQK_WAVE + (e % 4) * 16 + key % 16] = k_regs[n];
+        }
+    };
+    // turned latents (piece i: element i / 4, places 32 h + 8 (i % 4) on); what lies at places of positions beyond the
+    // tile's last token may be anything and is replaced by zero
+    auto fetch_turned = [&](int hp) {
+        const int page = max(0, pages[hp / 2]);
+        const bf16_t* vp = turned + (size_t)page * rk * TQK_PAGE + (hp & 1) * 32;
+        const bool edge = hp * 32 + 31 > pos_max;
+#pragma unroll
+        for (int n = 0; n < VP; ++n) {
+            const int i = threadIdx.x + n * 256;
+            const int col = i / 4, gq = i % 4;
+            lat_pack8 a;
+            a.q = *reinterpret_cast<const uint4*>(vp + (size_t)min(col, rk - 1) * TQK_PAGE + 8 * gq);
+            if (col >= rk) a.q = make_uint4(0, 0, 0, 0);
+            if (edge) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if ((hp / 2) * TQK_PAGE + value_position((hp & 1) * 32 + 8 * gq + e) > pos_max) a.u[e] = 0;
+            }
+            v_regs[n] = a.q;
+        }
+    };
+    auto store_turned = [&]() {
+#pragma unroll
+        for (int n = 0; n < VP; ++n) {
+            const int i = threadIdx.x + n * 256;
+            const int col = i / 4, gq = i % 4;
+            lds[(col / 16) * TQK_WAVE + gq * 16 + col % 16] = v_regs[n];
+        }
+    };
+
+    const int hp_first = lo_min / 32, hp_last = pos_max / 32;
+    fetch_rows(hp_first);
+    for (int hp = hp_first; hp <= hp_last; ++hp) {
+        const int kb = hp * 32;
+        store_rows();
+        __syncthreads();
+        fetch_turned(hp);
+        const bool mine = has && kb <= pos && kb + 31 >= lo;          // the half holds a position this wave's token sees
+        lat_pack8 pb;
+        float alpha = 1.f;
+        pb.q = make_uint4(0, 0, 0, 0);
+        if (mine) {
+            lat_floatx4_t s[2] = {lat_floatx4_t{0.f, 0.f, 0.f, 0.f}, lat_floatx4_t{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    lat_pack8 a;
+                    a.q = lds[(j * KS + ks) * TQK_WAVE + lane];
+                    s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, bq[ks].v, s[j], 0, 0, 0);
+                }
+            float p[2][4];
+            float mx = -INFINITY;
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int key = kb + 16 * j + 4 * g + i;
+                    p[j][i] = key >= lo && key <= pos ? s[j][i] * scale : -INFINITY;
+                    mx = fmaxf(mx, p[j][i]);
+                }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, TQK_WAVE));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, TQK_WAVE));
+            const float m_new = fmaxf(m, mx);               // finite: the half holds a visible position
+            alpha = expf(m - m_new);
+            float sum = 0.f;
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    p[j][i] = expf(p[j][i] - m_new);
+                    sum += p[j][i];
+                    pb.u[4 * j + i] = float_to_bf16_bits(p[j][i]);
+                }
+            sum += __shfl_xor(sum, 16, TQK_WAVE);
+            sum += __shfl_xor(sum, 32, TQK_WAVE);
+            l = l * alpha + sum;
+            m = m_new;
+        }
+        __syncthreads();                                    // every wave is done with the rows
+        store_turned();
+        __syncthreads();
+        if (hp < hp_last) fetch_rows(hp + 1);
+        if (mine) {
+#pragma unroll
+            for (int ct = 0; ct < NCT; ++ct) {
+                lat_pack8 a;
+                a.q = lds[ct * TQK_WAVE + lane];
+                o[ct] *= alpha;
+                o[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pb.v, o[ct], 0, 0, 0);
+            }
+        }
+        __syncthreads();                                    // every wave is done with the turned latents
+    }
+    if (!has || head >= n_heads) return;
+    float* dst = out + ((size_t)t * n_heads + head) * rk;
+    const float inv = 1.f / l;
+#pragma unroll
+    for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int col = 16 * ct + 4 * g + i;
+            if (col < rk) dst[col] = o[ct][i] * inv;
+        }
+}
+
 // ---- values ----------------------------------------------------------------------------------
 // A block: LAT_TT tokens of one head; a wave takes value columns in turn, its lanes share a row of
 // W_uv (contiguous loads) and their partial sums are added up in a fixed order.
@@ -514,6 +693,34 @@ extern "C" int tqk_latent_attention_mfma(const float* qa, const void* cache, con
         return tqk_check_launch("tqk_latent_attention_mfma merge");
     }
     return 0;
+}
+
+/* The same for steps that bring several tokens per sequence: tiles of up to 4 consecutive tokens of one sequence (tile i:
+ * sequence tile_seq[i], first packed token tile_tok0[i], tile_count[i] tokens), a block a tile. */
+extern "C" int tqk_latent_attention_tiles(const float* qa, const void* cache, const void* turned, const int32_t* tok_pos,
+                                          const int32_t* page_table, int table_width, int n_seqs, int n_pages, const int32_t* tile_seq,
+                                          const int32_t* tile_tok0, const int32_t* tile_count, int n_tiles, int window, float scale,
+                                          float* out, int n_tokens, int n_heads, int rk, int dr, void* stream) {
+    TQK_REQUIRE(qa && cache && turned && tok_pos && page_table && out && tile_seq && tile_tok0 && tile_count, "tqk_latent_attention_tiles: null pointer");
+    TQK_REQUIRE(n_tokens >= 0 && n_tiles >= 0 && n_heads > 0 && rk > 0 && dr >= 0, "tqk_latent_attention_tiles: bad sizes");
+    TQK_REQUIRE(tqk_latent_attention_mfma_supported(rk, dr), "tqk_latent_attention_tiles: a latent of %d + %d values is not taken", rk, dr);
+    TQK_REQUIRE(table_width > 0 && n_pages > 0 && n_seqs > 0 && window >= 0, "tqk_latent_attention_tiles: empty page table or negative window");
+    TQK_REQUIRE(((((uintptr_t)qa) | ((uintptr_t)cache) | ((uintptr_t)turned)) & 15) == 0, "tqk_latent_attention_tiles: operands must be 16-byte aligned");
+    if (n_tokens == 0 || n_tiles == 0) return 0;
+    const int dk = rk + dr;
+    dim3 grid(n_tiles, (n_heads + 15) / 16);
+    TQK_REQUIRE(grid.y <= 65535, "tqk_latent_attention_tiles: too many heads for the grid");
+    hipStream_t s = (hipStream_t)stream;
+#define TQK_LAT_TILE(KS, NCT)                                                                                                           \
+    latent_attention_tile_kernel<KS, NCT><<<grid, 4 * TQK_WAVE, 0, s>>>(qa, (const bf16_t*)cache, (const bf16_t*)turned, tok_pos, page_table, \
+                                                                        table_width, tile_seq, tile_tok0, tile_count, window, scale, out,    \
+                                                                        n_heads, rk, dk)
+    if (rk <= 128 && dk <= 160) TQK_LAT_TILE(5, 8);
+    else if (rk <= 256 && dk <= 320) TQK_LAT_TILE(10, 16);
+    else if (dk <= 576) TQK_LAT_TILE(18, 32);
+    else TQK_LAT_TILE(20, 32);
+#undef TQK_LAT_TILE
+    return tqk_check_launch("tqk_latent_attention_tiles");
 }
 
 extern "C" int tqk_latent_attention(const float* qa, const void* cache, int cache_dtype, const int32_t* tok_seq, const int32_t* tok_pos,

@@ -218,6 +218,11 @@ int tqk_latent_attention_mfma(const float* qa, const void* cache, const void* tu
                               const int32_t* page_table, int table_width, int n_seqs, int n_pages, int window, float scale,
                               float* out, int n_tokens, int n_heads, int rk, int dr, int n_parts, float* part_o, float* part_ml,
                               void* stream);
+/* the same for steps of several tokens per sequence: tiles of up to 4 consecutive tokens of one sequence, a block a tile */
+int tqk_latent_attention_tiles(const float* qa, const void* cache, const void* turned, const int32_t* tok_pos,
+                               const int32_t* page_table, int table_width, int n_seqs, int n_pages, const int32_t* tile_seq,
+                               const int32_t* tile_tok0, const int32_t* tile_count, int n_tiles, int window, float scale,
+                               float* out, int n_tokens, int n_heads, int rk, int dr, void* stream);
 /* y [tokens, heads * dv] = gate[t, h] * W_uv,h o[t, h] (w_uv [heads * dv, rk]; gate may be null) */
 int tqk_latent_values(const float* o, const void* w_uv, int w_dtype, const float* gate, int n_heads, int rk, int dv, void* y,
                       int y_dtype, int n_tokens, void* stream);

@@ -152,7 +152,8 @@ def latent_spec(m, hidden, eps, own=True, cache_window=None):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("shape", [(5, 24, 8, 40, 48, 56, 23), (1, 8, 2, 8, 16, 8, 1), (3, 10, 6, 14, 20, 18, 130), (2, 64, 32, 64, 96, 128, 64),
-                                   (4, 16, 8, 16, 32, 24, 65)])
+                                   (4, 16, 8, 16, 32, 24, 65), (2, 32, 64, 32, 64, 256, 70), (18, 32, 64, 32, 64, 512, 70),
+                                   (1, 32, 128, 32, 64, 512, 33)])         # the last three: the kernels' builds for larger latents
 def test_latent_attention_part(dtype, shape):
     """Two sequences in shared steps: one in two portions and then token by token, across a page border and past
     its window; the other whole.  A second mixer reads the first one's cache with a window of its own."""
@@ -185,8 +186,9 @@ def test_latent_attention_part(dtype, shape):
     for i in range(2):
         pos = torch.arange(xs[i].shape[0])
         kv = plain.latent_kv(xs[i].float(), w, "", m, eps, pos, low)
-        torch.testing.assert_close(torch.cat(got[i]).float().cpu(), plain.latent_attention(xs[i].float(), w, "", m, eps, pos, kv, low), **TOL[dtype])
-        torch.testing.assert_close(torch.cat(got2[i]).float().cpu(), plain.latent_attention(xs[i].float(), w2, "", m2, eps, pos, kv, low), **TOL[dtype])
+        # (rows against the outputs' own spread: sharpened scores carry bfloat16 rounding further than an absolute allowance fits)
+        N.close(torch.cat(got[i]), plain.latent_attention(xs[i].float(), w, "", m, eps, pos, kv, low), dtype, "own cache, sequence %d" % i, spare=0)
+        N.close(torch.cat(got2[i]), plain.latent_attention(xs[i].float(), w2, "", m2, eps, pos, kv, low), dtype, "read cache, sequence %d" % i, spare=0)
 
 
 # ---- whole models ----------------------------------------------------------------------------------------

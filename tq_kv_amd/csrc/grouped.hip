@@ -54,7 +54,12 @@ void grouped_mfma_kernel(GroupedArgs p) {
     // tiles of more than 16 rows: the block brings a step's rows of x into LDS once (one 16-byte piece a thread), in the
     // order the lanes take them, two buffers in turn with one barrier a step; its waves read them from there
     constexpr bool STAGE = RT > 1;
+    // tiles of up to 16 rows: the block's four waves take the same features and a quarter of K each (a wave alone would
+    // walk all of K with one load under way after the other), and add their sums up through LDS in the waves' order
+    constexpr bool SPLIT = RT == 1;
+    constexpr int NBK = GATED ? 2 : 1;
     __shared__ uint4 x_lds[STAGE ? 2 : 1][4][STAGE ? 16 * RT : 1];
+    __shared__ grp_floatx4_t sum_lds[SPLIT ? GRP_WAVES : 1][NBK][CB][SPLIT ? TQK_WAVE : 1];
     int group, row0, n_rows;
     if (p.tile_group) {
         const int tile = blockIdx.y;
@@ -69,9 +74,9 @@ void grouped_mfma_kernel(GroupedArgs p) {
     }
     const int wave = threadIdx.x / TQK_WAVE, lane = threadIdx.x % TQK_WAVE;
     const int g = lane / 16, r16 = lane % 16;
-    const int n0 = (blockIdx.x * GRP_WAVES + wave) * CB * 16;
+    const int n0 = (SPLIT ? blockIdx.x : blockIdx.x * GRP_WAVES + wave) * CB * 16;
     const bool active = n0 < p.N;
-    if (!STAGE && !active) return;
+    if (!STAGE && !SPLIT && !active) return;
     constexpr int NB = GATED ? 2 : 1;
     grp_floatx4_t acc[NB][RT][CB];
 #pragma unroll
@@ -141,10 +146,12 @@ void grouped_mfma_kernel(GroupedArgs p) {
     };
     grp_pack8 b_next[NB][CB];
     uint4 x_next = make_uint4(0, 0, 0, 0);
-    load_w(0, b_next);
+    load_w(min(SPLIT ? wave * (((p.K + 32 * GRP_WAVES - 1) / (32 * GRP_WAVES)) * 32) : 0, ((p.K - 1) / 32) * 32), b_next);
     if (STAGE) x_next = load_x(stage_off, 8 * stage_g);
-    const int k_last = ((p.K - 1) / 32) * 32;
-    for (int k0 = 0, step = 0; k0 < p.K; k0 += 32, ++step) {
+    const int k_quarter = SPLIT ? ((p.K + 32 * GRP_WAVES - 1) / (32 * GRP_WAVES)) * 32 : p.K;
+    const int k_begin = SPLIT ? wave * k_quarter : 0, k_end = SPLIT ? min(p.K, k_begin + k_quarter) : p.K;
+    const int k_last = k_end > k_begin ? ((k_end - 1 - k_begin) / 32) * 32 + k_begin : k_begin;
+    for (int k0 = k_begin, step = 0; k0 < k_end; k0 += 32, ++step) {
         grp_pack8 a[RT], b[NB][CB];
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
@@ -166,6 +173,19 @@ void grouped_mfma_kernel(GroupedArgs p) {
 #pragma unroll
                 for (int cb = 0; cb < CB; ++cb)
                     acc[nb][rt][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[rt].v, b[nb][cb].v, acc[nb][rt][cb], 0, 0, 0);
+    }
+    if (SPLIT) {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) sum_lds[SPLIT ? wave : 0][nb][cb][SPLIT ? lane : 0] = acc[nb][0][cb];
+        __syncthreads();
+        if (wave != 0) return;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb)
+                for (int w = 1; w < (SPLIT ? GRP_WAVES : 1); ++w) acc[nb][0][cb] += sum_lds[w][nb][cb][SPLIT ? lane : 0];
     }
     if (!active) return;
     // the lane holds, of each block, feature n0 + 16 cb + r16 of rows 16 rt + 4 g + i
@@ -202,7 +222,8 @@ static int launch_grouped(const GroupedArgs& a, int tiles, hipStream_t s) {
     // loaded serves many products; tiles of up to 16 rows stream the weights, 16 features a wave, 32 where there are many
     const int rt = a.tile_rows_max > 32 ? 4 : a.tile_rows_max > 16 ? 2 : 1;
     const int cb = rt > 1 ? (GATED ? 2 : (a.N >= 256 ? 4 : 2)) : (((long long)a.N / 16) * tiles >= 4096 && !GATED ? 2 : 1);
-    dim3 grid((a.N + GRP_WAVES * cb * 16 - 1) / (GRP_WAVES * cb * 16), tiles);
+    const int per_block = (rt == 1 ? 1 : GRP_WAVES) * cb * 16;       // tiles of up to 16 rows: the waves of a block share its features
+    dim3 grid((a.N + per_block - 1) / per_block, tiles);
 #define TQK_GRP(RT, CB) grouped_mfma_kernel<RT, CB, GATED><<<grid, GRP_WAVES * TQK_WAVE, 0, s>>>(a)
     if (rt == 4) { if (cb == 4) TQK_GRP(4, 4); else TQK_GRP(4, 2); }
     else if (rt == 2) { if (cb == 4) TQK_GRP(2, 4); else TQK_GRP(2, 2); }

@@ -358,21 +358,39 @@ void latent_attention_mfma_kernel(const float* __restrict__ qa, const bf16_t* __
 }
 
 // the parts of a (token, head) in their order: out = sum_p o_p e^(m_p - M) / sum_p l_p e^(m_p - M)
+#define LAT_MAX_PARTS 128
 __global__ __launch_bounds__(128)
 void latent_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml, int n_parts, int rk, float* __restrict__ out) {
+    __shared__ float wgt[LAT_MAX_PARTS];
+    __shared__ float total;
     const size_t row = blockIdx.x;
     const float* ml = part_ml + row * n_parts * 2;
+    // the parts' maxima and weights once, side by side, instead of one load after the other in every thread
+    const float mine = threadIdx.x < n_parts ? ml[2 * threadIdx.x] : -INFINITY;
+    const float mine_l = threadIdx.x < n_parts ? ml[2 * threadIdx.x + 1] : 0.f;
+    if (threadIdx.x < LAT_MAX_PARTS) wgt[threadIdx.x] = mine;
+    __syncthreads();
     float M = -INFINITY;
-    for (int p = 0; p < n_parts; ++p) M = fmaxf(M, ml[2 * p]);
-    float L = 0.f;
-    for (int p = 0; p < n_parts; ++p) L += ml[2 * p + 1] * expf(ml[2 * p] - M);
+    for (int p = 0; p < n_parts; ++p) M = fmaxf(M, wgt[p]);
+    __syncthreads();
+    if (threadIdx.x < LAT_MAX_PARTS) wgt[threadIdx.x] = threadIdx.x < n_parts ? expf(mine - M) : 0.f;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float L = 0.f;
+        for (int p = 0; p < n_parts; ++p) L += part_ml[(row * n_parts + p) * 2 + 1] * wgt[p];
+        total = L;
+    }
+    (void)mine_l;
+    __syncthreads();
+    const float inv = 1.f / total;
     for (int c = threadIdx.x; c < rk; c += blockDim.x) {
         float v = 0.f;
+#pragma unroll 8
         for (int p = 0; p < n_parts; ++p) {
-            const float wgt = expf(ml[2 * p] - M);
-            if (wgt > 0.f) v = fmaf(part_o[(row * n_parts + p) * rk + c], wgt, v);
+            const float x = part_o[(row * n_parts + p) * rk + c];
+            v = fmaf(wgt[p] > 0.f ? x : 0.f, wgt[p], v);        // a part without a page left its memory as it was
         }
-        out[row * rk + c] = v / L;
+        out[row * rk + c] = v * inv;
     }
 }
 
@@ -659,14 +677,15 @@ extern "C" int tqk_latent_attention_parts(int n_tokens, int n_heads, int table_w
     const long long items = (long long)n_tokens * ((n_heads + 15) / 16);
     const int pages = window > 0 ? std::min(table_width, (window + TQK_PAGE - 2) / TQK_PAGE + 1) : table_width;
     if (items >= 512 || pages <= 1) return 1;
-    return (int)std::max(1LL, std::min((long long)pages, 1024 / std::max(1LL, items)));
+    return (int)std::max(1LL, std::min(std::min((long long)pages, (long long)LAT_MAX_PARTS), 1024 / std::max(1LL, items)));
 }
 
 extern "C" int tqk_latent_attention_mfma(const float* qa, const void* cache, const void* turned, const int32_t* tok_seq, const int32_t* tok_pos,
                                          const int32_t* page_table, int table_width, int n_seqs, int n_pages, int window, float scale,
                                          float* out, int n_tokens, int n_heads, int rk, int dr, int n_parts, float* part_o, float* part_ml,
                                          void* stream) {
-    TQK_REQUIRE(n_parts >= 1 && (n_parts == 1 || (part_o && part_ml)), "tqk_latent_attention_mfma: %d parts without memory for them", n_parts);
+    TQK_REQUIRE(n_parts >= 1 && n_parts <= LAT_MAX_PARTS && (n_parts == 1 || (part_o && part_ml)),
+                "tqk_latent_attention_mfma: %d parts (1 to %d, with memory for them)", n_parts, LAT_MAX_PARTS);
     TQK_REQUIRE(qa && cache && turned && tok_seq && tok_pos && page_table && out, "tqk_latent_attention_mfma: null pointer");
     TQK_REQUIRE(n_tokens >= 0 && n_heads > 0 && rk > 0 && dr >= 0, "tqk_latent_attention_mfma: bad sizes");
     TQK_REQUIRE(tqk_latent_attention_mfma_supported(rk, dr), "tqk_latent_attention_mfma: a latent of %d + %d values is not taken", rk, dr);

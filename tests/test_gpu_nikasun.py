@@ -25,6 +25,11 @@ ROOT = os.path.join(os.path.dirname(os.path.abspath(__file__)), "..")
 DTYPES = ["float32", "bfloat16"]
 
 
+@pytest.fixture(autouse=True)
+def _seeded():
+    torch.manual_seed(1234)
+
+
 def load(part, tensors, dtype):
     part.load({k: v.to(DT[dtype]).to(DEV) for k, v in tensors.items()})
     return {k: v.to(DT[dtype]).float() for k, v in tensors.items()}
@@ -100,7 +105,12 @@ def test_routed_experts(dtype, experts, top, shared, rows):
     gain = {n: 1.5 for n in ff.tensors() if n.endswith("gate") or n.endswith("up")}
     gain["router"] = 4.0
     w = load(ff, rand_weights(ff, 3, gain), dtype)
-    x = torch.randn(rows, hidden).to(DT[dtype]).float()
+    # inputs whose router's choice does not hang on rounding: the first `rows` such of four times as many
+    cand = torch.randn(4 * rows + 8, hidden).to(DT[dtype]).float()
+    zc = (cand @ w["router"].T).sort(-1, descending=True).values
+    keep = torch.ones(cand.shape[0], dtype=torch.bool) if top == experts else (zc[:, top - 1] - zc[:, top]) > 0.1
+    x = cand[keep][:rows]
+    assert x.shape[0] == rows
     mlp = {"router": {"experts": experts, "top": top, "scale": 1.75}, "expert": {"ff": inter, "limit": 1.0},
            "shared": {"ff": 40, "limit": 2.0} if shared else None}
     want = plain.moe_ff(x, w, "", mlp, DT[dtype])

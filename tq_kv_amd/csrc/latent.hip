@@ -397,10 +397,9 @@ void latent_merge_kernel(const float* __restrict__ part_o, const float* __restri
 // ---- attention on the matrix cores, tiles of queries (prompts) -----------------------------------
 // A block of four waves takes up to four consecutive tokens of one sequence, a wave a token's 16 heads.  The products
 // are those of the kernel above; what differs is where the cache comes from: the block brings half a page (32
-// positions) of rows, then of turned latents, into LDS in the order the lanes take them, once for all four tokens, so
+// positions) of rows and of turned latents into LDS in the order the lanes take them, once for all four tokens, so
 // the cache is read a quarter as often.  A thread's pieces of the next half are asked for before the products on
-// this one and written to LDS after the barrier that ends them (rows while the second product runs, turned latents
-// while the first does).  The absorbed queries stay in registers.
+// this one and written to LDS after the barrier that ends them.  The absorbed queries stay in registers.
 template <int KS, int NCT>
 __global__ __launch_bounds__(4 * TQK_WAVE)
 void latent_attention_tile_kernel(const float* __restrict__ qa, const bf16_t* __restrict__ cache, const bf16_t* __restrict__ turned,
@@ -408,10 +407,10 @@ void latent_attention_tile_kernel(const float* __restrict__ qa, const bf16_t* __
                                   const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_tok0,
                                   const int32_t* __restrict__ tile_count, int window, float scale, float* __restrict__ out, int n_heads,
                                   int rk, int dk) {
-    constexpr int SLOTS = (2 * KS > NCT ? 2 * KS : NCT) * TQK_WAVE;
     constexpr int KP = (128 * KS + 255) / 256;          // 16-byte pieces of half a page of rows a thread brings
     constexpr int VP = NCT / 4;                         // and of turned latents
-    __shared__ uint4 lds[SLOTS];
+    __shared__ uint4 lds_k[2 * KS * TQK_WAVE];          // (together up to 72 KB of the 160 KB a compute unit has)
+    __shared__ uint4 lds_v[NCT * TQK_WAVE];
     const int tile = blockIdx.x;
     const int tok0 = tile_tok0[tile], count = min(4, tile_count[tile]);
     const int32_t* pages = page_table + (size_t)tile_seq[tile] * table_width;
@@ -444,39 +443,38 @@ void latent_attention_tile_kernel(const float* __restrict__ qa, const bf16_t* __
     for (int ct = 0; ct < NCT; ++ct) o[ct] = lat_floatx4_t{0.f, 0.f, 0.f, 0.f};
     float m = -INFINITY, l = 0.f;
 
-    // a thread's pieces of half a page: rows (piece i: position i / (4 KS) of the half, elements 8 (i % (4 KS)) on)
+    // A thread's pieces of half a page are those whose places in LDS follow one another from thread to thread (its
+    // writes to LDS then meet no bank twice); in memory a wave's pieces are 64 contiguous bytes of each of 16 rows.
     uint4 k_regs[KP], v_regs[VP];
     auto fetch_rows = [&](int hp) {
         const int page = max(0, pages[hp / 2]);
         const bf16_t* kp = cache + ((size_t)page * TQK_PAGE + (size_t)(hp & 1) * 32) * dk;
 #pragma unroll
         for (int n = 0; n < KP; ++n) {
-            const int i = threadIdx.x + n * 256;
-            const int key = min(i / (4 * KS), 31), e = i % (4 * KS);
-            const bool in = 8 * e + 8 <= dk;
-            k_regs[n] = *reinterpret_cast<const uint4*>(kp + (size_t)key * dk + (in ? 8 * e : 0));
+            const int slot = min((int)threadIdx.x + n * 256, 2 * KS * TQK_WAVE - 1);
+            const int j = slot / (KS * TQK_WAVE), ks = (slot / TQK_WAVE) % KS, ln = slot % TQK_WAVE;
+            const int key = 16 * j + ln % 16, e0 = 32 * ks + 8 * (ln / 16);
+            const bool in = e0 + 8 <= dk;
+            k_regs[n] = *reinterpret_cast<const uint4*>(kp + (size_t)key * dk + (in ? e0 : 0));
             if (!in) k_regs[n] = make_uint4(0, 0, 0, 0);
         }
     };
     auto store_rows = [&]() {
 #pragma unroll
         for (int n = 0; n < KP; ++n) {
-            const int i = threadIdx.x + n * 256;
-            if (i >= 128 * KS) continue;
-            const int key = i / (4 * KS), e = i % (4 * KS);
-            lds[((key / 16) * KS + e / 4) * TQK_WAVE + (e % 4) * 16 + key % 16] = k_regs[n];
+            const int slot = threadIdx.x + n * 256;
+            if (slot < 2 * KS * TQK_WAVE) lds_k[slot] = k_regs[n];
         }
     };
-    // turned latents (piece i: element i / 4, places 32 h + 8 (i % 4) on); what lies at places of positions beyond the
-    // tile's last token may be anything and is replaced by zero
+    // turned latents; what lies at places of positions beyond the tile's last token may be anything and is replaced by zero
     auto fetch_turned = [&](int hp) {
         const int page = max(0, pages[hp / 2]);
         const bf16_t* vp = turned + (size_t)page * rk * TQK_PAGE + (hp & 1) * 32;
         const bool edge = hp * 32 + 31 > pos_max;
 #pragma unroll
         for (int n = 0; n < VP; ++n) {
-            const int i = threadIdx.x + n * 256;
-            const int col = i / 4, gq = i % 4;
+            const int slot = threadIdx.x + n * 256;
+            const int col = 16 * (slot / TQK_WAVE) + slot % 16, gq = (slot % TQK_WAVE) / 16;
             lat_pack8 a;
             a.q = *reinterpret_cast<const uint4*>(vp + (size_t)min(col, rk - 1) * TQK_PAGE + 8 * gq);
             if (col >= rk) a.q = make_uint4(0, 0, 0, 0);
@@ -490,24 +488,23 @@ void latent_attention_tile_kernel(const float* __restrict__ qa, const bf16_t* __
     };
     auto store_turned = [&]() {
 #pragma unroll
-        for (int n = 0; n < VP; ++n) {
-            const int i = threadIdx.x + n * 256;
-            const int col = i / 4, gq = i % 4;
-            lds[(col / 16) * TQK_WAVE + gq * 16 + col % 16] = v_regs[n];
-        }
+        for (int n = 0; n < VP; ++n) lds_v[threadIdx.x + n * 256] = v_regs[n];
     };
 
     const int hp_first = lo_min / 32, hp_last = pos_max / 32;
     fetch_rows(hp_first);
+    fetch_turned(hp_first);
+    store_rows();
+    store_turned();
+    __syncthreads();
     for (int hp = hp_first; hp <= hp_last; ++hp) {
         const int kb = hp * 32;
-        store_rows();
-        __syncthreads();
-        fetch_turned(hp);
+        // the next half is asked for now and has this half's products to arrive
+        if (hp < hp_last) {
+            fetch_rows(hp + 1);
+            fetch_turned(hp + 1);
+        }
         const bool mine = has && kb <= pos && kb + 31 >= lo;          // the half holds a position this wave's token sees
-        lat_pack8 pb;
-        float alpha = 1.f;
-        pb.q = make_uint4(0, 0, 0, 0);
         if (mine) {
             lat_floatx4_t s[2] = {lat_floatx4_t{0.f, 0.f, 0.f, 0.f}, lat_floatx4_t{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
@@ -515,7 +512,7 @@ void latent_attention_tile_kernel(const float* __restrict__ qa, const bf16_t* __
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
                     lat_pack8 a;
-                    a.q = lds[(j * KS + ks) * TQK_WAVE + lane];
+                    a.q = lds_k[(j * KS + ks) * TQK_WAVE + lane];
                     s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, bq[ks].v, s[j], 0, 0, 0);
                 }
             float p[2][4];
@@ -531,8 +528,9 @@ void latent_attention_tile_kernel(const float* __restrict__ qa, const bf16_t* __
             mx = fmaxf(mx, __shfl_xor(mx, 16, TQK_WAVE));
             mx = fmaxf(mx, __shfl_xor(mx, 32, TQK_WAVE));
             const float m_new = fmaxf(m, mx);               // finite: the half holds a visible position
-            alpha = expf(m - m_new);
+            const float alpha = expf(m - m_new);
             float sum = 0.f;
+            lat_pack8 pb;
 #pragma unroll
             for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -545,21 +543,20 @@ void latent_attention_tile_kernel(const float* __restrict__ qa, const bf16_t* __
             sum += __shfl_xor(sum, 32, TQK_WAVE);
             l = l * alpha + sum;
             m = m_new;
-        }
-        __syncthreads();                                    // every wave is done with the rows
-        store_turned();
-        __syncthreads();
-        if (hp < hp_last) fetch_rows(hp + 1);
-        if (mine) {
 #pragma unroll
             for (int ct = 0; ct < NCT; ++ct) {
                 lat_pack8 a;
-                a.q = lds[ct * TQK_WAVE + lane];
+                a.q = lds_v[ct * TQK_WAVE + lane];
                 o[ct] *= alpha;
                 o[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pb.v, o[ct], 0, 0, 0);
             }
         }
-        __syncthreads();                                    // every wave is done with the turned latents
+        __syncthreads();                                    // every wave is done with this half
+        if (hp < hp_last) {
+            store_rows();
+            store_turned();
+        }
+        __syncthreads();
     }
     if (!has || head >= n_heads) return;
     float* dst = out + ((size_t)t * n_heads + head) * rk;

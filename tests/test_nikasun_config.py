@@ -161,3 +161,17 @@ def test_plain_layers_that_share_a_cache_and_layers_without_feed_forward():
     assert "l1.norm2" not in w and base.shape == (50, cfg["vocab"]) and torch.isfinite(base).all()
     # causal
     torch.testing.assert_close(plain.forward(w, cfg, toks[:20]), base[:20], atol=1e-5, rtol=1e-5)
+
+
+def test_more_windows_than_cache_groups_share_the_largest():
+    """Twenty layers with windows of their own: caches of equal row size then keep the largest window, each layer still
+    sees its own."""
+    cfg = N.config(64, 32, [(N.mixer(2, 8, 8, 8, 16, 24, 10 + 3 * i), N.dense(16)) for i in range(20)])
+    spec = spec_from_dict(cfg)
+    mixers = [l.block.params["mixer"].params for l in spec.layers]
+    assert {m["cache_window"] for m in mixers} == {67} and [m["window"] for m in mixers] == [10 + 3 * i for i in range(20)]
+    engine = Engine(Model.random(cfg, seed=0, dtype="float32", device="cpu"), max_tokens=10 * PAGE, max_slots=2)
+    assert len(engine.cache.kv_groups) == 1
+    # with few windows every cache keeps its own
+    few = N.config(64, 32, [(N.mixer(2, 8, 8, 8, 16, 24, w), None) for w in (5, 70, 5)])
+    assert [l.block.params["mixer"].params["cache_window"] for l in spec_from_dict(few).layers] == [5, 70, 5]

@@ -159,6 +159,23 @@ ModelSpec nikasun_spec(const Json& c) {
         if (m["window"].is_null()) keep_all[owner] = true;
         else keep[owner] = std::max(keep[owner], (long long)m["window"].as_int());
     }
+    // Caches of equal row size and window are one group of the cache, and the cache's bookkeeping takes TQE_MAX_GROUPS of
+    // them.  A model with more different windows than that keeps, in caches of equal row size, the largest of their
+    // windows (what a layer sees is its own window still).
+    auto row_of = [&](size_t l) { return std::make_pair(layers[l]["mixer"]["kv_rank"].as_int(), layers[l]["mixer"]["rot_dim"].as_int()); };
+    std::vector<std::vector<long long>> distinct;
+    for (size_t l = 0; l < layers.size(); ++l) {
+        if (!layers[l]["mixer"]["kv_from"].is_null()) continue;
+        const std::vector<long long> key = {row_of(l).first, row_of(l).second, keep_all[l] ? -1 : keep[l]};
+        if (std::find(distinct.begin(), distinct.end(), key) == distinct.end()) distinct.push_back(key);
+    }
+    if ((int)distinct.size() > TQE_MAX_GROUPS)
+        for (size_t l = 0; l < layers.size(); ++l)
+            for (size_t o = 0; o < layers.size(); ++o)
+                if (layers[l]["mixer"]["kv_from"].is_null() && layers[o]["mixer"]["kv_from"].is_null() && row_of(l) == row_of(o)) {
+                    keep[l] = std::max(keep[l], keep[o]);
+                    if (keep_all[o]) keep_all[l] = true;
+                }
     ModelSpec s;
     s.architecture = "Nikasun";
     s.vocab_size = c["vocab"].as_int();

@@ -357,6 +357,142 @@ void latent_attention_mfma_kernel(const float* __restrict__ qa, const bf16_t* __
     }
 }
 
+// ---- attention on the matrix cores, a block per (token, 16 heads, part) (decoding) -------------------
+// The same products as latent_attention_mfma_kernel, shared out over the four waves of a block so that no wave has a
+// long chain of loads to wait for: wave j takes the scores of the page's keys 16 j .. 16 j + 15 (a quarter of the rows),
+// the waves exchange their maxima, sums and probabilities through LDS, and wave w takes a quarter of the latent's
+// elements in the second product.  The absorbed queries wait in LDS for all four.
+template <int KS, int NCT>
+__global__ __launch_bounds__(4 * TQK_WAVE)
+void latent_attention_page_kernel(const float* __restrict__ qa, const bf16_t* __restrict__ cache, const bf16_t* __restrict__ turned,
+                                  const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos,
+                                  const int32_t* __restrict__ page_table, int table_width, int window, float scale,
+                                  float* __restrict__ out, int n_heads, int n_chunks, int rk, int dk, int n_parts,
+                                  float* __restrict__ part_o, float* __restrict__ part_ml) {
+    constexpr int CT = NCT / 4;                         // 16-element blocks of the latent a wave takes
+    __shared__ uint4 q_lds[KS][TQK_WAVE];
+    __shared__ float mx_lds[4][16], sum_lds[4][16];
+    __shared__ uint2 p_lds[4][TQK_WAVE];
+    const int wave = threadIdx.x / TQK_WAVE, lane = threadIdx.x % TQK_WAVE;
+    const int g = lane / 16, r16 = lane % 16;
+    const int item = blockIdx.x;
+    const int part = item % n_parts;
+    const int t = (item / n_parts) / n_chunks, chunk = (item / n_parts) % n_chunks;
+    const int head = chunk * 16 + r16;
+    const int pos = tok_pos[t];
+    const int32_t* pages = page_table + (size_t)tok_seq[t] * table_width;
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    for (int i = threadIdx.x; i < KS * TQK_WAVE; i += 4 * TQK_WAVE) {
+        const int ks = i / TQK_WAVE, ln = i % TQK_WAVE;
+        const int h = chunk * 16 + ln % 16, e0 = 32 * ks + 8 * (ln / 16);
+        lat_pack8 bq;
+        bq.q = make_uint4(0, 0, 0, 0);
+        if (h < n_heads && e0 + 8 <= dk) {
+            const float4* src = reinterpret_cast<const float4*>(qa + ((size_t)t * n_heads + h) * dk + e0);
+            const float4 a = src[0], b = src[1];
+            bq.u[0] = float_to_bf16_bits(a.x); bq.u[1] = float_to_bf16_bits(a.y);
+            bq.u[2] = float_to_bf16_bits(a.z); bq.u[3] = float_to_bf16_bits(a.w);
+            bq.u[4] = float_to_bf16_bits(b.x); bq.u[5] = float_to_bf16_bits(b.y);
+            bq.u[6] = float_to_bf16_bits(b.z); bq.u[7] = float_to_bf16_bits(b.w);
+        }
+        q_lds[ks][ln] = bq.q;
+    }
+    __syncthreads();
+    lat_floatx4_t o[CT];
+#pragma unroll
+    for (int c = 0; c < CT; ++c) o[c] = lat_floatx4_t{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+
+    for (int kb = (lo / TQK_PAGE + part) * TQK_PAGE; kb <= pos; kb += TQK_PAGE * n_parts) {
+        const int page = max(0, pages[kb / TQK_PAGE]);
+        const bf16_t* kp = cache + ((size_t)page * TQK_PAGE + 16 * wave + r16) * dk;
+        const bf16_t* vp = turned + (size_t)page * rk * TQK_PAGE;
+        lat_floatx4_t s = lat_floatx4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const int e0 = 32 * ks + 8 * g;
+            const bool in = e0 + 8 <= dk;
+            lat_pack8 a, bq;
+            a.q = *reinterpret_cast<const uint4*>(kp + (in ? e0 : dk - 8));
+            if (!in) a.q = make_uint4(0, 0, 0, 0);
+            bq.q = q_lds[ks][lane];
+            s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, bq.v, s, 0, 0, 0);
+        }
+        float p[4];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int key = kb + 16 * wave + 4 * g + i;
+            p[i] = key >= lo && key <= pos ? s[i] * scale : -INFINITY;
+            mx = fmaxf(mx, p[i]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, TQK_WAVE));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, TQK_WAVE));
+        if (g == 0) mx_lds[wave][r16] = mx;
+        __syncthreads();
+        const float m_new = fmaxf(fmaxf(m, fmaxf(mx_lds[0][r16], mx_lds[1][r16])), fmaxf(mx_lds[2][r16], mx_lds[3][r16]));   // finite
+        const float alpha = expf(m - m_new);
+        float sum = 0.f;
+        lat_pack8 mine;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            p[i] = expf(p[i] - m_new);
+            sum += p[i];
+            mine.u[i] = float_to_bf16_bits(p[i]);
+        }
+        sum += __shfl_xor(sum, 16, TQK_WAVE);
+        sum += __shfl_xor(sum, 32, TQK_WAVE);
+        if (g == 0) sum_lds[wave][r16] = sum;
+        p_lds[wave][lane] = make_uint2(mine.q.x, mine.q.y);
+        __syncthreads();
+        l = l * alpha + ((sum_lds[0][r16] + sum_lds[1][r16]) + (sum_lds[2][r16] + sum_lds[3][r16]));
+        m = m_new;
+        lat_pack8 pb[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const uint2 first = p_lds[2 * h][lane], second = p_lds[2 * h + 1][lane];
+            pb[h].q = make_uint4(first.x, first.y, second.x, second.y);
+        }
+        const bool edge = kb < lo || kb + TQK_PAGE - 1 > pos;
+#pragma unroll
+        for (int c = 0; c < CT; ++c) {
+            const int col = 16 * (wave * CT + c) + r16;
+            const int colc = min(col, rk - 1);
+            o[c] *= alpha;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                lat_pack8 a;
+                a.q = *reinterpret_cast<const uint4*>(vp + (size_t)colc * TQK_PAGE + 32 * h + 8 * g);
+                if (col >= rk) a.q = make_uint4(0, 0, 0, 0);
+                if (edge) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const int key = kb + value_position(32 * h + 8 * g + e);
+                        if (key < lo || key > pos) a.u[e] = 0;
+                    }
+                }
+                o[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pb[h].v, o[c], 0, 0, 0);
+            }
+        }
+        __syncthreads();                                // the next page writes the exchanged values again
+    }
+    if (head >= n_heads) return;
+    float* dst = n_parts > 1 ? part_o + (((size_t)t * n_heads + head) * n_parts + part) * rk : out + ((size_t)t * n_heads + head) * rk;
+    const float inv = n_parts > 1 ? 1.f : 1.f / l;
+#pragma unroll
+    for (int c = 0; c < CT; ++c)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int col = 16 * (wave * CT + c) + 4 * g + i;
+            if (col < rk) dst[col] = o[c][i] * inv;
+        }
+    if (n_parts > 1 && wave == 0 && g == 0) {
+        float* ml = part_ml + (((size_t)t * n_heads + head) * n_parts + part) * 2;
+        ml[0] = m;
+        ml[1] = l;
+    }
+}
+
 // the parts of a (token, head) in their order: out = sum_p o_p e^(m_p - M) / sum_p l_p e^(m_p - M)
 #define LAT_MAX_PARTS 128
 __global__ __launch_bounds__(128)
@@ -698,10 +834,17 @@ extern "C" int tqk_latent_attention_mfma(const float* qa, const void* cache, con
         qa, (const bf16_t*)cache, (const bf16_t*)turned, tok_seq, tok_pos, page_table, table_width, window, scale, out, n_tokens, n_heads, \
         n_chunks, rk, dk, n_parts, part_o, part_ml)
     // the smallest build that holds the row and the latent (steps and blocks beyond the sizes multiply zeros)
-    if (rk <= 128 && dk <= 160) TQK_LAT_MFMA(5, 8, 4);
-    else if (rk <= 256 && dk <= 320) TQK_LAT_MFMA(10, 16, 4);
-    else if (dk <= 576) TQK_LAT_MFMA(18, 32, 2);
-    else TQK_LAT_MFMA(20, 32, 2);
+    // a block of four waves per (token, 16 heads, part) wherever that leaves the chip enough blocks; a wave each otherwise
+#define TQK_LAT_PAGE(KS, NCT)                                                                                                          \
+    latent_attention_page_kernel<KS, NCT><<<(unsigned)items, 4 * TQK_WAVE, 0, s>>>(qa, (const bf16_t*)cache, (const bf16_t*)turned, tok_seq, \
+                                                                                   tok_pos, page_table, table_width, window, scale, out,    \
+                                                                                   n_heads, n_chunks, rk, dk, n_parts, part_o, part_ml)
+    const bool by_block = items <= 16384;
+    if (rk <= 128 && dk <= 160) { if (by_block) TQK_LAT_PAGE(5, 8); else TQK_LAT_MFMA(5, 8, 4); }
+    else if (rk <= 256 && dk <= 320) { if (by_block) TQK_LAT_PAGE(10, 16); else TQK_LAT_MFMA(10, 16, 4); }
+    else if (dk <= 576) { if (by_block) TQK_LAT_PAGE(18, 32); else TQK_LAT_MFMA(18, 32, 2); }
+    else { if (by_block) TQK_LAT_PAGE(20, 32); else TQK_LAT_MFMA(20, 32, 2); }
+#undef TQK_LAT_PAGE
 #undef TQK_LAT_MFMA
     if (tqk_check_launch("tqk_latent_attention_mfma")) return -1;
     if (n_parts > 1) {

@@ -16,7 +16,7 @@
 #include "tq_kernels.h"
 
 #define MOE_MAX_EXPERTS 512
-#define MOE_ROUTE_WAVES 4
+#define MOE_ROUTE_WAVES 8
 #define MOE_TM 32               // rows of a tile
 #define MOE_TN 64               // features of a block
 #define MOE_TK 16               // k per stage
@@ -208,11 +208,19 @@ template <typename TA>
 __global__ __launch_bounds__(256)
 void moe_combine_kernel(const TA* __restrict__ y, const int32_t* __restrict__ pair_pos, const float* __restrict__ weight, int top,
                         const TA* __restrict__ shared, TA* __restrict__ out, int hidden) {
+    // the token's rows and weights once, side by side, not one load after the other in front of every element
+    __shared__ int32_t row[MOE_MAX_EXPERTS];
+    __shared__ float wt[MOE_MAX_EXPERTS];
     const int t = blockIdx.x;
+    for (int k = threadIdx.x; k < top; k += blockDim.x) {
+        row[k] = pair_pos[(size_t)t * top + k];
+        wt[k] = weight[(size_t)t * top + k];
+    }
+    __syncthreads();
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
         float v = 0.f;
-        for (int k = 0; k < top; ++k)
-            v = fmaf(weight[(size_t)t * top + k], to_float(y[(size_t)pair_pos[(size_t)t * top + k] * hidden + i]), v);
+#pragma unroll 4
+        for (int k = 0; k < top; ++k) v = fmaf(wt[k], to_float(y[(size_t)row[k] * hidden + i]), v);
         if (shared) v += to_float(shared[(size_t)t * hidden + i]);
         out[(size_t)t * hidden + i] = from_float<TA>(v);
     }
@@ -290,7 +298,7 @@ extern "C" int tqk_moe_product(const void* x, int act_dtype, const int32_t* x_ro
 extern "C" int tqk_moe_combine(const void* y, int act_dtype, const int32_t* pair_pos, const float* weight, int top, const void* shared, void* out,
                                int n_tokens, int hidden, void* stream) {
     TQK_REQUIRE(y && pair_pos && weight && out, "tqk_moe_combine: null pointer");
-    TQK_REQUIRE(top > 0 && hidden > 0 && n_tokens >= 0, "tqk_moe_combine: bad sizes");
+    TQK_REQUIRE(top > 0 && top <= MOE_MAX_EXPERTS && hidden > 0 && n_tokens >= 0, "tqk_moe_combine: bad sizes");
     if (n_tokens == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     if (act_dtype == TQK_F32)

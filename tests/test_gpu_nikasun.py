@@ -92,7 +92,7 @@ def test_gated_feed_forward(dtype, rows, gate):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("experts,top,shared", [(6, 2, True), (1, 1, False), (5, 5, False), (70, 3, True)])
-@pytest.mark.parametrize("rows", [1, 11, 150])
+@pytest.mark.parametrize("rows", [1, 11, 150, 700])         # tiles of 16, 32 and 64 rows, one and many an expert
 def test_routed_experts(dtype, experts, top, shared, rows):
     env = BuildEnv(DEV, DT[dtype])
     hidden, inter = 80, 24
@@ -345,6 +345,20 @@ def test_far_keys_among_hundreds(dtype, tmp_path_factory):
         seen = N.row_errors(run_cut(eng, changed, c)[329:], run_cut(eng, toks, c)[329:]).item()
         noise = 0.0 if dtype == "float32" else 0.02
         assert seen > 0 and 0.5 * moved - noise < seen < 2.0 * moved + noise
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_long_prompt_in_one_step_and_in_two(dtype, tmp_path_factory):
+    """Several hundred tokens in a step: the products per head and per expert run over many of their largest tiles."""
+    cfg, w, eng = engine("mixed", dtype, tmp_path_factory, 1.0)
+    toks = N.tokens(530, cfg["vocab"], 321)
+    want = N.plain_logits(cfg, w, toks)
+    whole = run_cut(eng, toks, [])
+    N.close(whole, want, dtype, "530 tokens in one step")
+    two = run_cut(eng, toks, [270])
+    N.close(two, want, dtype, "530 tokens in two steps")
+    if dtype == "float32":
+        assert torch.equal(two, whole)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -1,0 +1,218 @@
+// Attention whose heads have values of another size than their keys, with what some designs put
+// around the softmax: a norm of every query and key head before the rotation, values mixed with
+// those of an earlier layer, a cap on the scores, a window that keeps a sequence's first
+// positions, and a sink in the softmax's denominator.  float32 arithmetic throughout, any sizes;
+// the kernels for the matrix cores are in attention_masked_mfma.hip.
+//
+//   q_h <- rot(q_h / rms(q_h) * w_q),  k_g <- rot(k_g / rms(k_g) * w_k)      (rms with eps inside the root)
+//   v_g <- (1 - lambda) v_g + lambda v'_g                                      (v' another layer's values of the token)
+//   s_ij = scale q_i . k_j;  s_ij <- cap tanh(s_ij / cap)
+//   i sees j  iff  j <= i and (window == 0 or i - j < window or j < keep_first)
+//   p_ij = exp(s_ij) / (sum_j' exp(s_ij') + exp(sink_h))
+//
+// Cache pages: keys [kv head][position][key_dim], values [kv head][value_dim][place of the position]
+// (value_place in common.h).
+#include "common.h"
+#include "tq_kernels.h"
+
+#define AM_WAVES 4
+#define AM_MAX_D 256
+
+// ---- norm of heads, rotation, value mixing, cache write ---------------------------------------------
+// A wave per head of a token: heads 0..H-1 are queries, then G key heads, then G value heads; a row of qkv is
+// [H * dk | G * dk | G * dv].
+template <typename TA, typename TW>
+__global__ __launch_bounds__(AM_WAVES * TQK_WAVE)
+void normed_rope_store_kernel(const TA* __restrict__ qkv, const TW* __restrict__ q_norm_w, const TW* __restrict__ k_norm_w, float eps,
+                              const float* __restrict__ cos_table, const float* __restrict__ sin_table, int rot_dim, int max_positions,
+                              const TW* __restrict__ mix, const TA* __restrict__ mix_with, TA* __restrict__ mix_keep,
+                              const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos,
+                              const int32_t* __restrict__ page_table, int table_width, TA* __restrict__ keys, TA* __restrict__ values,
+                              TA* __restrict__ q_out, int n_heads, int n_kv_heads, int dk, int dv, int write_kv) {
+    const int t = blockIdx.x;
+    const int head = blockIdx.y * AM_WAVES + threadIdx.x / TQK_WAVE;
+    const int lane = threadIdx.x % TQK_WAVE;
+    if (head >= n_heads + 2 * n_kv_heads) return;
+    const int pos = tok_pos[t];
+    const int kind = head < n_heads ? 0 : (head < n_heads + n_kv_heads ? 1 : 2);
+    if (kind != 0 && !write_kv) return;
+    const size_t total = (size_t)(n_heads + n_kv_heads) * dk + (size_t)n_kv_heads * dv;
+    const TA* row = qkv + (size_t)t * total;
+    int page = -1;
+    if (kind != 0) {
+        page = page_table[(size_t)tok_seq[t] * table_width + pos / TQK_PAGE];
+        if (page < 0) return;                          // the host never lets this happen
+    }
+    if (kind == 2) {
+        const int g = head - n_heads - n_kv_heads;
+        const TA* src = row + (size_t)(n_heads + n_kv_heads) * dk + (size_t)g * dv;
+        TA* dst = values + ((size_t)page * n_kv_heads + g) * TQK_PAGE * dv + value_place(pos % TQK_PAGE);
+        const float lam = mix && mix_with ? to_float(mix[0]) : 0.f;
+        for (int i = lane; i < dv; i += TQK_WAVE) {
+            float v = to_float(src[i]);
+            const size_t at = ((size_t)t * n_kv_heads + g) * dv + i;
+            if (mix_with) v = (1.f - lam) * v + lam * to_float(mix_with[at]);
+            const TA stored = from_float<TA>(v);
+            if (mix_keep) mix_keep[at] = stored;
+            dst[(size_t)i * TQK_PAGE] = stored;
+        }
+        return;
+    }
+    const TA* src = row + (size_t)head * dk;
+    const TW* w = kind == 0 ? q_norm_w : k_norm_w;
+    float inv = 1.f;
+    if (w) {
+        float ss = 0.f;
+        for (int i = lane; i < dk; i += TQK_WAVE) { const float v = to_float(src[i]); ss = fmaf(v, v, ss); }
+        inv = 1.f / sqrtf(wave_sum(ss) / (float)dk + eps);
+    }
+    TA* dst = kind == 0 ? q_out + ((size_t)t * n_heads + head) * dk
+                        : keys + (((size_t)page * n_kv_heads + (head - n_heads)) * TQK_PAGE + pos % TQK_PAGE) * dk;
+    const int half = rot_dim / 2;
+    const bool rotate = rot_dim > 0 && pos < max_positions;
+    for (int i = lane; i < dk; i += TQK_WAVE) {
+        float x = to_float(src[i]) * inv * (w ? to_float(w[i]) : 1.f);
+        if (rotate && i < rot_dim) {
+            const bool first = i < half;
+            const int p = first ? i : i - half, partner = first ? i + half : i - half;
+            const float y = to_float(src[partner]) * inv * (w ? to_float(w[partner]) : 1.f);
+            const float c = cos_table[(size_t)pos * half + p], s = sin_table[(size_t)pos * half + p];
+            x = first ? x * c - y * s : x * c + y * s;
+        }
+        dst[i] = from_float<TA>(x);
+    }
+}
+
+// ---- attention, a wave per (token, head) --------------------------------------------------------------
+// Keys are taken a page at a time; lane j computes the score of key j of the page, the softmax runs online over the
+// pages, then lane c accumulates output element c (+64, ...).  The order of operations for a query depends on its
+// position alone.  Pages all of whose positions are hidden (between the kept first positions and the window) are
+// passed over and may have been given back.
+template <typename T, typename TS>
+__global__ __launch_bounds__(AM_WAVES * TQK_WAVE)
+void attention_masked_kernel(const T* __restrict__ q, const T* __restrict__ keys, const T* __restrict__ values,
+                             const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos,
+                             const int32_t* __restrict__ page_table, int table_width, int window, int keep_first, float scale, float cap,
+                             const TS* __restrict__ sink, T* __restrict__ out, int n_tokens, int n_heads, int n_kv_heads, int dk, int dv) {
+    __shared__ float q_lds[AM_WAVES][AM_MAX_D];
+    const int wave = threadIdx.x / TQK_WAVE, lane = threadIdx.x % TQK_WAVE;
+    const int t = blockIdx.x * AM_WAVES + wave;
+    const int head = blockIdx.y;
+    const bool live = t < n_tokens;
+    if (live) {
+        const T* qv = q + ((size_t)t * n_heads + head) * dk;
+        for (int i = lane; i < dk; i += TQK_WAVE) q_lds[wave][i] = to_float(qv[i]);
+    }
+    __syncthreads();
+    if (!live) return;
+
+    const int pos = tok_pos[t];
+    const int32_t* pages = page_table + (size_t)tok_seq[t] * table_width;
+    const int kvh = head / (n_heads / n_kv_heads);
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int kept = window > 0 ? keep_first : 0;
+    const float* qf = q_lds[wave];
+
+    constexpr int NACC = AM_MAX_D / TQK_WAVE;
+    float acc[NACC];
+#pragma unroll
+    for (int i = 0; i < NACC; ++i) acc[i] = 0.f;
+    // the sink is a key of score sink_h without a value: the running maximum and sum start from it
+    float m = sink ? to_float(sink[head]) : -INFINITY, l = sink ? 1.f : 0.f;
+
+    for (int kb = 0; kb <= pos; kb += TQK_PAGE) {
+        if (kb + TQK_PAGE <= lo && kb >= kept) continue;
+        const int page = pages[kb / TQK_PAGE];
+        const int j = kb + lane;
+        const bool valid = j <= pos && (j >= lo || j < kept) && page >= 0;
+        const size_t pg = (size_t)(page < 0 ? 0 : page) * n_kv_heads + kvh;
+        float s = -INFINITY;
+        if (valid) {
+            const T* kr = keys + (pg * TQK_PAGE + lane) * dk;
+            float dot = 0.f;
+            for (int i = 0; i < dk; ++i) dot = fmaf(qf[i], to_float(kr[i]), dot);
+            s = dot * scale;
+            if (cap > 0.f) s = cap * tanhf(s / cap);
+        }
+        const float m_new = fmaxf(m, wave_max(s));     // finite: the page holds at least one visible key, or the sink came first
+        const float p = valid ? expf(s - m_new) : 0.f;
+        const float alpha = expf(m - m_new);            // exp(-inf) = 0 on the first page
+        l = l * alpha + wave_sum(p);
+        m = m_new;
+        const int n_keys = min(TQK_PAGE, pos - kb + 1);
+        const T* vb = values + pg * TQK_PAGE * dv;
+#pragma unroll
+        for (int a = 0; a < NACC; ++a) {
+            const int c = lane + a * TQK_WAVE;
+            float sum = acc[a] * alpha;
+            if (a * TQK_WAVE < dv) {
+                for (int jj = 0; jj < n_keys; ++jj) {
+                    const float pj = __shfl(p, jj, TQK_WAVE);
+                    if (c < dv && pj != 0.f) sum = fmaf(pj, to_float(vb[(size_t)c * TQK_PAGE + value_place(jj)]), sum);
+                }
+            }
+            acc[a] = sum;
+        }
+    }
+    T* o = out + ((size_t)t * n_heads + head) * dv;
+#pragma unroll
+    for (int a = 0; a < NACC; ++a) {
+        const int c = lane + a * TQK_WAVE;
+        if (c < dv) o[c] = from_float<T>(acc[a] / l);
+    }
+}
+
+extern "C" int tqk_normed_rope_store(const void* qkv, int act_dtype, const void* q_norm_w, const void* k_norm_w, int w_dtype, float eps,
+                                     const float* cos_table, const float* sin_table, int rot_dim, int max_positions, const void* mix,
+                                     const void* mix_with, void* mix_keep, const int32_t* tok_seq, const int32_t* tok_pos,
+                                     const int32_t* page_table, int table_width, void* keys, void* values, void* q_out, int n_tokens,
+                                     int n_heads, int n_kv_heads, int key_dim, int value_dim, int write_kv, void* stream) {
+    TQK_REQUIRE(qkv && tok_pos && q_out, "tqk_normed_rope_store: null pointer");
+    TQK_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && key_dim > 0 && value_dim > 0, "tqk_normed_rope_store: bad sizes");
+    TQK_REQUIRE(rot_dim >= 0 && rot_dim % 2 == 0 && rot_dim <= key_dim, "tqk_normed_rope_store: rot_dim %d must be even and <= key_dim %d", rot_dim, key_dim);
+    TQK_REQUIRE(rot_dim == 0 || (cos_table && sin_table && max_positions > 0), "tqk_normed_rope_store: rotation without tables");
+    TQK_REQUIRE(!write_kv || (tok_seq && page_table && keys && values && table_width > 0), "tqk_normed_rope_store: no cache to write to");
+    TQK_REQUIRE(!mix_with || mix, "tqk_normed_rope_store: values to mix with, but no weight");
+    if (n_tokens == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    dim3 grid(n_tokens, (n_heads + 2 * n_kv_heads + AM_WAVES - 1) / AM_WAVES);
+#define TQK_NRS(TA, TW) \
+    normed_rope_store_kernel<TA, TW><<<grid, AM_WAVES * TQK_WAVE, 0, s>>>((const TA*)qkv, (const TW*)q_norm_w, (const TW*)k_norm_w, eps, cos_table, sin_table, \
+        rot_dim, max_positions, (const TW*)mix, (const TA*)mix_with, (TA*)mix_keep, tok_seq, tok_pos, page_table, table_width, (TA*)keys, (TA*)values, \
+        (TA*)q_out, n_heads, n_kv_heads, key_dim, value_dim, write_kv)
+    if (act_dtype == TQK_F32 && w_dtype == TQK_F32) TQK_NRS(float, float);
+    else if (act_dtype == TQK_F32 && w_dtype == TQK_BF16) TQK_NRS(float, bf16_t);
+    else if (act_dtype == TQK_BF16 && w_dtype == TQK_F32) TQK_NRS(bf16_t, float);
+    else if (act_dtype == TQK_BF16 && w_dtype == TQK_BF16) TQK_NRS(bf16_t, bf16_t);
+    else return tqk_fail("tqk_normed_rope_store: unknown dtypes %d, %d", act_dtype, w_dtype);
+#undef TQK_NRS
+    return tqk_check_launch("tqk_normed_rope_store");
+}
+
+extern "C" int tqk_attention_masked_max_dim(void) { return AM_MAX_D; }
+
+extern "C" int tqk_attention_masked(const void* q, const void* keys, const void* values, int act_dtype, const int32_t* tok_seq,
+                                    const int32_t* tok_pos, const int32_t* page_table, int table_width, int n_seqs, int n_pages, int window,
+                                    int keep_first, float scale, float cap, const void* sink, int sink_dtype, void* out, int n_tokens,
+                                    int n_heads, int n_kv_heads, int key_dim, int value_dim, void* stream) {
+    TQK_REQUIRE(q && keys && values && tok_seq && tok_pos && page_table && out, "tqk_attention_masked: null pointer");
+    TQK_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && key_dim > 0 && value_dim > 0, "tqk_attention_masked: bad sizes");
+    TQK_REQUIRE(n_heads % n_kv_heads == 0, "tqk_attention_masked: %d heads are not a multiple of %d kv heads", n_heads, n_kv_heads);
+    TQK_REQUIRE(key_dim <= AM_MAX_D && value_dim <= AM_MAX_D, "tqk_attention_masked: head sizes %d and %d, the kernel takes up to %d", key_dim, value_dim, AM_MAX_D);
+    TQK_REQUIRE(n_heads <= 65535, "tqk_attention_masked: too many heads for the grid");
+    TQK_REQUIRE(table_width > 0 && n_pages > 0 && n_seqs > 0, "tqk_attention_masked: empty page table");
+    TQK_REQUIRE(window >= 0 && keep_first >= 0 && cap >= 0.f, "tqk_attention_masked: negative window, kept positions or cap");
+    if (n_tokens == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    dim3 grid((n_tokens + AM_WAVES - 1) / AM_WAVES, n_heads);
+#define TQK_AM(T, TS) \
+    attention_masked_kernel<T, TS><<<grid, AM_WAVES * TQK_WAVE, 0, s>>>((const T*)q, (const T*)keys, (const T*)values, tok_seq, tok_pos, page_table, \
+        table_width, window, keep_first, scale, cap, (const TS*)sink, (T*)out, n_tokens, n_heads, n_kv_heads, key_dim, value_dim)
+    if (act_dtype == TQK_F32 && (!sink || sink_dtype == TQK_F32)) TQK_AM(float, float);
+    else if (act_dtype == TQK_F32 && sink_dtype == TQK_BF16) TQK_AM(float, bf16_t);
+    else if (act_dtype == TQK_BF16 && (!sink || sink_dtype == TQK_BF16)) TQK_AM(bf16_t, bf16_t);
+    else if (act_dtype == TQK_BF16 && sink_dtype == TQK_F32) TQK_AM(bf16_t, float);
+    else return tqk_fail("tqk_attention_masked: unknown dtypes %d, %d", act_dtype, sink_dtype);
+#undef TQK_AM
+    return tqk_check_launch("tqk_attention_masked");
+}

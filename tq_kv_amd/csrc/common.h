@@ -69,9 +69,12 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
 //   TQK_GATE_RELU     max(g, 0) u
 //   TQK_GATE_CLAMPED  g' sigmoid(alpha g') (u' + 1) with g' = min(g, limit), u' = clamp(u, -limit, limit)
 //   TQK_GATE_GELU     gelu_tanh(g) u
-enum { TQK_GATE_SILU = 0, TQK_GATE_RELU = 1, TQK_GATE_CLAMPED = 2, TQK_GATE_GELU = 3, TQK_GATE_KINDS = 4 };
+//   TQK_GATE_RELU2    max(g, 0)^2 u
+// A feed-forward without a gate product applies the same function to its one product, with u = 1 (act_value).
+enum { TQK_GATE_SILU = 0, TQK_GATE_RELU = 1, TQK_GATE_CLAMPED = 2, TQK_GATE_GELU = 3, TQK_GATE_RELU2 = 4, TQK_GATE_KINDS = 5 };
 __device__ __forceinline__ float gate_value(int kind, float limit, float alpha, float g, float u) {
     if (kind == TQK_GATE_RELU) return fmaxf(g, 0.f) * u;
+    if (kind == TQK_GATE_RELU2) { const float r = fmaxf(g, 0.f); return r * r * u; }
     if (kind == TQK_GATE_CLAMPED) {
         g = fminf(g, limit);
         u = fminf(fmaxf(u, -limit), limit);
@@ -80,6 +83,8 @@ __device__ __forceinline__ float gate_value(int kind, float limit, float alpha, 
     if (kind == TQK_GATE_GELU) return 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))) * u;
     return (g / (1.f + expf(-g))) * u;
 }
+
+__device__ __forceinline__ float act_value(int kind, float limit, float alpha, float z) { return gate_value(kind, limit, alpha, z, 1.f); }
 
 // ---- host side ------------------------------------------------------------------
 enum { TQK_F32 = 0, TQK_BF16 = 1 };

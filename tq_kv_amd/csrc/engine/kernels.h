@@ -67,10 +67,20 @@ TQ_QUERY(int, moe_tile_rows);
 TQ_QUERY(int, grouped_supported, int);
 TQ_KERNEL(moe_product_mfma, cptr, ci32, cptr, long long, void*, int, int, int, int, float, float, ci32, ci32, ci32, ci32, int, int, void*);
 TQ_KERNEL(head_product, cptr, int, long long, long long, cptr, void*, int, long long, long long, cf32, int, int, int, int, void*);
-TQ_KERNEL(moe_route, cptr, int, cptr, int, int, int, int, float, int32_t*, float*, int, void*);
+TQ_KERNEL(moe_route, cptr, int, cptr, int, int, int, int, float, int, int32_t*, float*, int, void*);
 TQ_KERNEL(moe_group, ci32, int, int, int, int, int32_t*, int32_t*, int32_t*, int32_t*, int32_t*, int32_t*, void*);
 TQ_KERNEL(moe_product, cptr, int, ci32, cptr, int, long long, void*, int, int, int, int, float, float, ci32, ci32, ci32, ci32, int, void*);
-TQ_KERNEL(moe_combine, cptr, int, ci32, cf32, int, cptr, void*, int, int, void*);
+TQ_KERNEL(moe_combine, cptr, int, ci32, cf32, int, cptr, cf32, void*, int, int, void*);
+TQ_KERNEL(pair_embed, cptr, int, int, long long, long long, ci32, ci32, ci32, ci32, ci32, ci32, float*, int, int, int, void*);
+TQ_KERNEL(remember_tokens, ci32, ci32, ci32, ci32, int32_t*, int, void*);
+TQ_KERNEL(norm_add, float*, cptr, int, cptr, int, float, void*, int, int, void*);
+TQ_KERNEL(unary_act, cptr, void*, int, long long, int, float, float, void*);
+TQ_KERNEL(row_gate, cptr, int, cptr, int, float*, int, int, void*);
+TQ_KERNEL(normed_rope_store, cptr, int, cptr, cptr, int, float, cf32, cf32, int, int, cptr, cptr, void*, ci32, ci32, ci32, int, void*, void*, void*,
+          int, int, int, int, int, int, void*);
+TQ_QUERY(int, attention_masked_max_dim);
+TQ_KERNEL(attention_masked, cptr, cptr, cptr, int, ci32, ci32, ci32, int, int, int, int, int, float, float, cptr, int, void*, int, int, int, int,
+          int, void*);
 TQ_QUERY(int, argmax_scratch_floats, int, int);
 TQ_KERNEL(argmax, cf32, int, int, int32_t*, float*, void*);
 TQ_KERNEL(repeat_penalty, float*, int, int, ci32, ci32, ci32, int, ci32, int, float, void*);

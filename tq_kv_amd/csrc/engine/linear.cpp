@@ -40,7 +40,9 @@ int mid_max_rows() {
     return n;
 }
 
-OwnedPtr make_owned(int dtype, const std::vector<int64_t>& dims) {
+OwnedPtr make_owned(int dtype, const std::vector<int64_t>& dims_given) {
+    // a scalar (no dimensions) is held as one element
+    const std::vector<int64_t> dims = dims_given.empty() ? std::vector<int64_t>{1} : dims_given;
     OwnedPtr o = std::make_shared<Owned>();
     o->t.dtype = dtype;
     o->t.ndim = (int)dims.size();
@@ -208,7 +210,8 @@ Gate Gate::from_params(const KeyReader& r, const char* what) {
     else if (name == "relu") g.kind = ReLU;
     else if (name == "clamped") g.kind = Clamped;
     else if (name == "gelu_tanh") g.kind = GELU;
-    else raise(TQE_ERR_ARGUMENT, "%s: unknown gate '%s' (known: silu, relu, clamped, gelu_tanh)", what, name.c_str());
+    else if (name == "relu2") g.kind = ReLU2;
+    else raise(TQE_ERR_ARGUMENT, "%s: unknown gate '%s' (known: silu, relu, clamped, gelu_tanh, relu2)", what, name.c_str());
     if (g.kind == Clamped) {
         g.limit = (float)r.number("limit", true);
         g.alpha = (float)r.number_or("alpha", 1.0, true);

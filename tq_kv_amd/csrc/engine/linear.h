@@ -66,9 +66,10 @@ struct Product {
 Product linear(StepContext& c, const Tensor& x, const Weight& w, const Tensor* bias, int out_dtype, bool leave_sums = false, Tensor* out = nullptr);
 // Which gate a gated feed-forward applies to its gate and up products g and u (the kernels' TQK_GATE_* codes):
 // silu g sigmoid(g) u; relu max(g, 0) u; clamped g' sigmoid(alpha g') (u' + 1) with g' = min(g, limit) and
-// u' = clamp(u, -limit, limit); gelu gelu_tanh(g) u.
+// u' = clamp(u, -limit, limit); gelu gelu_tanh(g) u; relu2 max(g, 0)^2 u.  A feed-forward without a gate product applies the
+// same function to its one product, with u = 1.
 struct Gate {
-    enum Kind { SiLU = 0, ReLU = 1, Clamped = 2, GELU = 3 };
+    enum Kind { SiLU = 0, ReLU = 1, Clamped = 2, GELU = 3, ReLU2 = 4 };
     int kind = SiLU;
     float limit = 0.f, alpha = 1.f;
     static Gate from_params(const KeyReader& r, const char* what);      // "gate" (default "silu"), "limit", "alpha"

@@ -30,6 +30,14 @@ Model::Model(const ModelSpec& s, int dtype_, bool on_gpu_) : spec(s), dtype(dtyp
         if (run.cache_of >= 0)
             if (Mixer* m = blocks_[(size_t)run.layer]->mixer()) m->reads_other_cache = true;
     }
+    // a part that acts on the stream may keep a state per sequence: one more entry of the cache, after the runs'
+    if (stream_position_ && stream_position_->stream_state_need().kind != CacheNeed::None) {
+        if (stream_position_->stream_state_need().kind != CacheNeed::State)
+            raise(TQE_ERR_ARGUMENT, "position kind '%s' asks for cache pages; a part that acts on the stream can keep a state only", spec.stream_position.kind.c_str());
+        stream_state_entry_ = (int)needs.size();
+        needs.push_back(stream_position_->stream_state_need());
+        cache_of.push_back(-1);
+    }
     // a step can be captured as a graph if every part's forward launches the same kernels whatever
     // the step's data are
     graph_safe = final_norm_->graph_safe && (!stream_position_ || stream_position_->graph_safe);
@@ -135,7 +143,7 @@ Tensor Model::forward(StepContext& c, const CacheStore& cache, float* out) {
     if (c.fuse_small) {
         stream.xw_buffer = c.alloc(BF16, {c.n_tokens, s.hidden_size});
         stream.ss_buffer = c.alloc(F32, {(s.hidden_size + 15) / 16, 16});        // the most pieces a product gives
-        const Norm* norm = firsts[0]->foldable() ? firsts[0] : nullptr;
+        const Norm* norm = firsts[0] && firsts[0]->foldable() ? firsts[0] : nullptr;
         K::embed(table.data, table.dtype, c.dev.tokens, c.n_tokens, (int)s.hidden_size, (int)s.vocab_size, scale, (float*)h.data,
                  stream.xw_buffer.data, norm ? norm->fold_weight()->data : nullptr, (float*)stream.ss_buffer.data, c.stream);
         stream.xw_for = norm;
@@ -145,7 +153,8 @@ Tensor Model::forward(StepContext& c, const CacheStore& cache, float* out) {
                  nullptr, c.stream);
     }
     if (stream_position_) {
-        stream_position_->add_to_stream(c, h);
+        if (stream_state_entry_ >= 0) stream_position_->add_to_stream_with(c, h, cache.entry(stream_state_entry_));
+        else stream_position_->add_to_stream(c, h);
         stream.invalidate();            // what the gather prepared for the first norm is of the stream before this
     }
     Stream* cur = &stream;

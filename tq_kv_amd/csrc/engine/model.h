@@ -43,6 +43,7 @@ private:
     std::vector<std::shared_ptr<Block>> blocks_;
     std::shared_ptr<Norm> final_norm_;
     std::shared_ptr<Position> stream_position_;
+    int stream_state_entry_ = -1;               // the cache entry of the stream position's state, if it keeps one
     OwnedPtr embedding_, head_bias_;
     Weight head_;
     Tensor head_logits(StepContext& c, Stream& stream, float* out);

@@ -101,7 +101,9 @@ struct Stream {
     int n_ss = 0;
     Norm* next_norm = nullptr;
     bool of_last_rows = false;
-    void invalidate() { xw_for = nullptr; }
+    Tensor copy;                        // h in the activation type, where a kernel that added to h also wrote it (valid while copy_valid)
+    bool copy_valid = false;
+    void invalidate() { xw_for = nullptr; copy_valid = false; }
 };
 
 // ---- building --------------------------------------------------------------------------------
@@ -149,6 +151,8 @@ public:
     virtual int64_t size() const = 0;
 };
 
+struct CacheEntry;
+
 enum RotaryStyle { STYLE_NONE = 0, STYLE_HALVES = 1, STYLE_PAIRS = 2 };
 
 class Position : public Part {
@@ -162,6 +166,10 @@ public:
     virtual void apply(StepContext& c, Tensor& q, Tensor& k, int64_t row_stride) { (void)c; (void)q; (void)k; (void)row_stride; }
     virtual bool acts_on_stream() const { return false; }
     virtual void add_to_stream(StepContext& c, Tensor& h) { (void)c; (void)h; }
+    // A part that acts on the stream may keep a fixed-size state per sequence (what it needs of a sequence's earlier
+    // steps): it names the need, and is then called with its state's cache entry instead.
+    virtual CacheNeed stream_state_need() const { return CacheNeed(); }
+    virtual void add_to_stream_with(StepContext& c, Tensor& h, const CacheEntry& state) { (void)state; add_to_stream(c, h); }
 };
 
 // What a mixer sees of the cache for one run of the order.
@@ -172,6 +180,7 @@ struct CacheEntry {
     Tensor state;                   // state: [slots, shape...]; row `slot` is a sequence's
     bool writes = true;             // false: reads another run's cache
     int window = 0;
+    int keep_first = 0;
 };
 
 class Mixer : public Part {
@@ -217,5 +226,6 @@ template <typename T> std::shared_ptr<T> build(const char* category, const PartS
 void register_builtin_parts();          // idempotent
 void register_latent_parts();           // parts_latent.cpp; called by register_builtin_parts
 void register_moe_parts();              // parts_moe.cpp; likewise
+void register_stream_parts();           // parts_stream.cpp; likewise
 
 }  // namespace tq

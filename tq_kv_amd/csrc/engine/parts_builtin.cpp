@@ -232,6 +232,16 @@ public:
 // query sees, itself included), scale (null: 1/sqrt(head_dim)), position (a part spec); optional
 // prompt_tile: queries per tile of the prompt kernel (16, 32, 64 or 128).
 //
+// What other designs put around the same attention, all off unless given: value_dim (a head's values are of another
+// size than its keys); qk_norm with eps (every query and key head is divided by its root mean square and multiplied
+// by a weight of head_dim values, before the rotation); cap (scores become cap tanh(s / cap)); keep_first (with a
+// window: a sequence's first positions stay visible, at their true places); sink (a learned number per head whose
+// exponential joins the softmax's denominator, with no key and no value); value_mix "source" (the values of the
+// step's tokens are handed to later layers) or "mixed" (v <- (1 - lambda) v + lambda v_source with a learned scalar,
+// before the cache); value_mix_key (which source, "values" unless given); names: the tensors' names inside the
+// part's prefix {q, k, v, o, q_norm, k_norm, sink, mix}.  With any of them the step runs through the kernels of
+// attention_masked.hip.
+//
 // Its pages: keys [kv heads, page, head_dim]; values [kv heads, head_dim, page], transposed inside
 // a page and the page's positions in the order the matrix cores take them (the kernels' own
 // layout, which is why the mixer names the shapes and the cache only multiplies them out).
@@ -252,6 +262,28 @@ public:
         if (r.has("window") && window_ < 1) raise(TQE_ERR_ARGUMENT, "attention: window must be at least 1, got %d", window_);
         scale_ = r.has("scale") ? (float)r.number("scale") : (float)(1.0 / sqrt((double)head_dim_));
         prompt_tile_ = r.has("prompt_tile") ? (int)r.integer("prompt_tile") : 0;
+        value_dim_ = r.has("value_dim") ? (int)r.integer("value_dim", 1) : head_dim_;
+        qk_norm_ = r.boolean_or("qk_norm", false);
+        eps_ = qk_norm_ ? (float)r.number("eps") : 0.f;
+        cap_ = r.has("cap") ? (float)r.number("cap", true) : 0.f;
+        keep_first_ = (int)r.integer_or("keep_first", 0, 0);
+        has_sink_ = r.boolean_or("sink", false);
+        const std::string mixing = r.string_or("value_mix", "none");
+        if (mixing == "none") value_mix_ = MIX_NONE;
+        else if (mixing == "source") value_mix_ = MIX_SOURCE;
+        else if (mixing == "mixed") value_mix_ = MIX_MIXED;
+        else raise(TQE_ERR_ARGUMENT, "attention: unknown value_mix '%s' (known: none, source, mixed)", mixing.c_str());
+        mix_key_ = "attention." + r.string_or("value_mix_key", "values");
+        if (keep_first_ > 0 && window_ == 0) raise(TQE_ERR_ARGUMENT, "attention: keep_first %d without a window", keep_first_);
+        extras_ = value_dim_ != head_dim_ || qk_norm_ || cap_ > 0.f || keep_first_ > 0 || has_sink_ || value_mix_ != MIX_NONE;
+        if (extras_ && (qkv_bias_ || out_bias_)) raise(TQE_ERR_ARGUMENT, "attention: biases go with none of value_dim, qk_norm, cap, keep_first, sink, value_mix");
+        {
+            const Json& names = spec.params["names"];
+            auto name = [&](const char* role, const char* fallback) { return names[role].is_string() ? names[role].as_string() : std::string(fallback); };
+            n_q_ = name("q", "q_proj.weight"); n_k_ = name("k", "k_proj.weight"); n_v_ = name("v", "v_proj.weight"); n_o_ = name("o", "o_proj.weight");
+            n_q_norm_ = name("q_norm", "q_norm.weight"); n_k_norm_ = name("k_norm", "k_norm.weight");
+            n_sink_ = name("sink", "sink"); n_mix_ = name("mix", "value_mix");
+        }
         if (r.has("prompt_tile") && prompt_tile_ != 16 && prompt_tile_ != 32 && prompt_tile_ != 64 && prompt_tile_ != 128)
             raise(TQE_ERR_ARGUMENT, "attention: prompt_tile must be 16, 32, 64 or 128, got %d", prompt_tile_);
         // what no attention kernel takes is refused here, before any weight is read
@@ -259,6 +291,9 @@ public:
         if (head_dim_ > max_d)
             raise(TQE_ERR_CONFIG, "attention: head_dim %d is more than the attention kernels take (%d)", head_dim_, max_d);
         if (n_heads_ > 65535) raise(TQE_ERR_CONFIG, "attention: %d heads are more than the attention kernels take (65535)", n_heads_);
+        if (extras_ && std::max(head_dim_, value_dim_) > K::attention_masked_max_dim.raw())
+            raise(TQE_ERR_CONFIG, "attention: heads of %d and %d values are more than the attention kernels take (%d)", head_dim_, value_dim_,
+                  K::attention_masked_max_dim.raw());
         const PartSpec pos = PartSpec::from_json(spec.params["position"], "attention: position");
         const std::string key = "position:" + pos.key();
         auto it = env.shared.find(key);
@@ -267,14 +302,29 @@ public:
         if (!position_) raise(TQE_ERR_ARGUMENT, "attention: part kind '%s' is no position", pos.kind.c_str());
         graph_safe = !position_->has_apply() || position_->graph_safe;
         takes_rows = true;
+        if (extras_) {
+            const Position::Tables tb = position_->tables();
+            if (position_->has_apply() || (tb.style != STYLE_NONE && (tb.style != STYLE_HALVES || tb.rot_dim > head_dim_)))
+                raise(TQE_ERR_ARGUMENT, "attention: with value_dim, qk_norm, cap, keep_first, sink or value_mix the position part must turn in halves from tables");
+        }
     }
 
     TensorSpecs tensors() const override {
         const int64_t q = (int64_t)n_heads_ * head_dim_, kv = (int64_t)n_kv_heads_ * head_dim_;
         auto w = [](int64_t a, int64_t b) { TensorSpec t; t.shape = {a, b}; return t; };
         auto b = [](int64_t a) { TensorSpec t; t.shape = {a}; return t; };
-        TensorSpecs t = {{"q_proj.weight", w(q, hidden_)}, {"k_proj.weight", w(kv, hidden_)}, {"v_proj.weight", w(kv, hidden_)},
-                         {"o_proj.weight", w(hidden_, q)}};
+        TensorSpecs t = {{n_q_, w(q, hidden_)}, {n_k_, w(kv, hidden_)}, {n_v_, w((int64_t)n_kv_heads_ * value_dim_, hidden_)},
+                         {n_o_, w(hidden_, (int64_t)n_heads_ * value_dim_)}};
+        if (qk_norm_) {
+            TensorSpec n = b(head_dim_);
+            n.init = "one_plus_normal";
+            n.std_dev = 0.1;
+            t.push_back({n_q_norm_, n});
+            t.push_back({n_k_norm_, n});
+        }
+        if (has_sink_) { TensorSpec s = b(n_heads_); s.std_dev = 1.0; t.push_back({n_sink_, s}); }
+        // the source layer of a mix has the scalar too, and does not use it
+        if (value_mix_ != MIX_NONE) { TensorSpec s; s.shape = {}; s.std_dev = 0.3; t.push_back({n_mix_, s}); }
         if (qkv_bias_) { t.push_back({"q_proj.bias", b(q)}); t.push_back({"k_proj.bias", b(kv)}); t.push_back({"v_proj.bias", b(kv)}); }
         if (out_bias_) t.push_back({"o_proj.bias", b(hidden_)});
         return t;
@@ -283,11 +333,14 @@ public:
     static OwnedPtr stacked(const std::vector<OwnedPtr>& parts, hipStream_t stream) { return stack_rows(parts, stream); }
 
     void load(Loaded& t, hipStream_t stream) override {
-        OwnedPtr qkv = stacked({take(t, "q_proj.weight"), take(t, "k_proj.weight"), take(t, "v_proj.weight")}, stream);
+        OwnedPtr qkv = stacked({take(t, n_q_.c_str()), take(t, n_k_.c_str()), take(t, n_v_.c_str())}, stream);
+        if (qk_norm_) { q_norm_ = take(t, n_q_norm_.c_str()); k_norm_ = take(t, n_k_norm_.c_str()); }
+        if (has_sink_) sink_ = take(t, n_sink_.c_str());
+        if (value_mix_ != MIX_NONE) mix_ = take(t, n_mix_.c_str());
         if (qkv_bias_) b_qkv_ = stacked({take(t, "q_proj.bias"), take(t, "k_proj.bias"), take(t, "v_proj.bias")}, stream);
         if (out_bias_) b_o_ = take(t, "o_proj.bias");
         w_qkv_ = make_weight(qkv, 1, false, stream);
-        w_o_ = make_weight(take(t, "o_proj.weight"), 1, b_o_ != nullptr, stream);
+        w_o_ = make_weight(take(t, n_o_.c_str()), 1, b_o_ != nullptr, stream);
     }
     OwnedPtr held(const std::string& name) const override {
         if (name == "qkv.weight") return w_qkv_.rows;
@@ -295,27 +348,32 @@ public:
         if (name == "qkv.bias") return b_qkv_;
         if (name == "o_proj.weight") return w_o_.rows;
         if (name == "o_proj.weight.packed") return w_o_.packed;
+        if (qk_norm_ && name == n_q_norm_) return q_norm_;
+        if (qk_norm_ && name == n_k_norm_) return k_norm_;
+        if (has_sink_ && name == n_sink_) return sink_;
+        if (value_mix_ != MIX_NONE && name == n_mix_) return mix_;
         return nullptr;
     }
     const char* trace_name() const override { return "attn"; }             // the reference's span, src/models/turbo_generic.rs:1920
     void product_shapes(std::vector<std::pair<int64_t, int64_t>>& out) const override {
-        out.push_back({(int64_t)(n_heads_ + 2 * n_kv_heads_) * head_dim_, hidden_});
-        out.push_back({hidden_, (int64_t)n_heads_ * head_dim_});
+        out.push_back({(int64_t)(n_heads_ + n_kv_heads_) * head_dim_ + (int64_t)n_kv_heads_ * value_dim_, hidden_});
+        out.push_back({hidden_, (int64_t)n_heads_ * value_dim_});
     }
 
     CacheNeed cache_need() const override {
         CacheNeed n;
         n.kind = CacheNeed::Pages;
         n.key_page = {n_kv_heads_, TQE_PAGE, head_dim_};
-        n.value_page = {n_kv_heads_, head_dim_, TQE_PAGE};
+        n.value_page = {n_kv_heads_, value_dim_, TQE_PAGE};
         n.window = window_;
+        n.keep_first = keep_first_;
         return n;
     }
 
     // The folded q/k/v kernel takes decoding steps (row m is sequence m) of rotary positions in the
     // halves layout over the whole head.
     bool fused_qkv_ok(const StepContext& c) const {
-        if (!(c.all_decode && fusable(c.n_tokens, w_qkv_) && head_dim_ % 32 == 0)) return false;
+        if (extras_ || !(c.all_decode && fusable(c.n_tokens, w_qkv_) && head_dim_ % 32 == 0)) return false;
         if (position_->has_apply()) return false;
         const Position::Tables tb = position_->tables();
         if (tb.style != STYLE_HALVES || tb.rot_dim != head_dim_) return false;
@@ -333,7 +391,10 @@ public:
         const StepContext::Table& table = c.tables.at((size_t)entry.group);
         Tensor q = c.alloc(dtype, {n, n_heads_, head_dim_});
         const int n_pages = (int)entry.keys.shape[0];
-        if (x.lazy || (c.fuse_small && entry.writes && fused_qkv_ok(c))) {
+        if (extras_) {
+            if (x.lazy) raise(TQE_ERR_STATE, "attention: this configuration takes no folded norm");
+            normed_qkv(c, x.x, entry, table, q);
+        } else if (x.lazy || (c.fuse_small && entry.writes && fused_qkv_ok(c))) {
             if (x.lazy && !entry.writes) raise(TQE_ERR_STATE, "a run that reads another run's cache cannot take a folded norm");
             const Position::Tables tb = position_->tables();
             const Tensor& xin = x.lazy ? x.norm.xw : x.x;
@@ -346,7 +407,7 @@ public:
         } else {
             qkv(c, x.x, entry, table, q);
         }
-        const int64_t qd = (int64_t)n_heads_ * head_dim_;
+        const int64_t qd = (int64_t)n_heads_ * value_dim_;
         if (last_rows) {
             if (c.n_last == 0) return Tensor(nullptr, dtype, {0, hidden_});
             Tensor ql = c.alloc(dtype, {c.n_last, n_heads_, head_dim_});
@@ -365,6 +426,45 @@ public:
     }
 
 private:
+    // product, then the heads' norm, rotation, value mixing and cache write in one kernel
+    void normed_qkv(StepContext& c, const Tensor& x, const CacheEntry& entry, const StepContext::Table& table, Tensor& q) {
+        const int64_t n = x.shape[0];
+        Product p = linear(c, x, w_qkv_, nullptr, x.dtype);
+        const Position::Tables tb = position_->tables();
+        const bool turn = tb.style != STYLE_NONE;
+        const int64_t vd = (int64_t)n_kv_heads_ * value_dim_;
+        const void* mix_with = nullptr;
+        void* mix_keep = nullptr;
+        if (value_mix_ == MIX_SOURCE && entry.writes) {
+            Tensor kept(c.ws->alloc_for_step((size_t)(n * vd) * dtype_size(x.dtype)), x.dtype, {n, vd});
+            c.carried[mix_key_] = kept;
+            mix_keep = kept.data;
+        } else if (value_mix_ == MIX_MIXED && entry.writes) {
+            auto it = c.carried.find(mix_key_);
+            if (it == c.carried.end()) raise(TQE_ERR_STATE, "attention: values are to be mixed with those of an earlier layer, and none has left any in this step");
+            if (it->second.dtype != x.dtype || it->second.shape[0] != n || it->second.shape[1] != vd)
+                raise(TQE_ERR_STATE, "attention: the values an earlier layer left are %s, wanted [%lld, %lld]", it->second.describe().c_str(), (long long)n, (long long)vd);
+            mix_with = it->second.data;
+        }
+        const int w_dtype = q_norm_ ? q_norm_->t.dtype : mix_ ? mix_->t.dtype : x.dtype;
+        if ((q_norm_ && k_norm_->t.dtype != w_dtype) || (mix_ && mix_->t.dtype != w_dtype))
+            raise(TQE_ERR_STATE, "attention: the heads' norm weights and the mixing scalar are of different types");
+        const bool write = entry.writes;
+        K::normed_rope_store(p.t.data, p.t.dtype, q_norm_ ? q_norm_->t.data : nullptr, k_norm_ ? k_norm_->t.data : nullptr, w_dtype, eps_,
+                             turn ? (const float*)tb.cos.data : nullptr, turn ? (const float*)tb.sin.data : nullptr, turn ? tb.rot_dim : 0,
+                             turn ? (int)tb.cos.shape[0] : 0, mix_ ? mix_->t.data : nullptr, mix_with, mix_keep, c.dev.tok_seq, c.dev.tok_pos,
+                             write ? table.dev : nullptr, write ? table.width : 0, write ? entry.keys.data : nullptr, write ? entry.values.data : nullptr,
+                             q.data, (int)n, n_heads_, n_kv_heads_, head_dim_, value_dim_, write ? 1 : 0, c.stream);
+    }
+
+    // attention of rows (sequence tok_seq[r], position tok_pos[r]) with the cap, the kept first positions and the sink
+    void attend_masked(StepContext& c, const Tensor& q, const CacheEntry& entry, const StepContext::Table& table, const int32_t* tok_seq,
+                       const int32_t* tok_pos, Tensor& out) {
+        K::attention_masked(q.data, entry.keys.data, entry.values.data, q.dtype, tok_seq, tok_pos, table.dev, table.width, c.n_seqs,
+                            (int)entry.keys.shape[0], window_, keep_first_, scale_, cap_, sink_ ? sink_->t.data : nullptr, sink_ ? sink_->t.dtype : 0,
+                            out.data, (int)q.shape[0], n_heads_, n_kv_heads_, head_dim_, value_dim_, c.stream);
+    }
+
     // queries per tile of the prompt kernel for this step
     int tile_for(StepContext& c) const {
         if (prompt_tile_) return prompt_tile_;
@@ -448,6 +548,7 @@ private:
     // tiled prompt kernel.
     void attend(StepContext& c, const Tensor& q, const CacheEntry& entry, const StepContext::Table& table, Tensor& out) {
         const int n = (int)q.shape[0], n_pages = (int)entry.keys.shape[0];
+        if (extras_) return attend_masked(c, q, entry, table, c.dev.tok_seq, c.dev.tok_pos, out);
         if (q.dtype == BF16 && c.all_decode && policy().decode_mfma && K::attention_decode_supported.raw(head_dim_))
             return decode_kernel(c, q, entry, c.dev.tok_pos, table.dev, table.width, out);
         // (not for steps of one token per sequence: tiles of one query are what the plain kernel does anyway,
@@ -468,6 +569,7 @@ private:
     // keys and values of all the step's tokens.
     void attend_rows(StepContext& c, const Tensor& q, const CacheEntry& entry, const StepContext::Table& table, Tensor& out) {
         const int n = (int)q.shape[0], n_pages = (int)entry.keys.shape[0];
+        if (extras_) return attend_masked(c, q, entry, table, c.dev.last_seq, c.dev.last_pos, out);
         if (q.dtype == BF16 && policy().decode_mfma && K::attention_decode_supported.raw(head_dim_) && c.n_last <= DECODE_KERNEL_ROWS) {
             // few rows: the decoding kernel shares a row's keys out over many blocks, where the prompt
             // kernel would walk them in one; a row is a sequence of its own to it
@@ -493,9 +595,14 @@ private:
     int n_heads_, n_kv_heads_, head_dim_, window_, prompt_tile_;
     bool qkv_bias_, out_bias_;
     float scale_;
+    enum { MIX_NONE = 0, MIX_SOURCE = 1, MIX_MIXED = 2 };
+    int value_dim_, keep_first_, value_mix_ = MIX_NONE;
+    bool qk_norm_ = false, has_sink_ = false, extras_ = false;
+    float eps_ = 0.f, cap_ = 0.f;
+    std::string mix_key_, n_q_, n_k_, n_v_, n_o_, n_q_norm_, n_k_norm_, n_sink_, n_mix_;
     std::shared_ptr<Position> position_;
     Weight w_qkv_, w_o_;
-    OwnedPtr b_qkv_, b_o_;
+    OwnedPtr b_qkv_, b_o_, q_norm_, k_norm_, sink_, mix_;
 };
 
 // ---- gated feed-forward ----------------------------------------------------------------------------
@@ -746,6 +853,7 @@ void register_builtin_parts() {
         register_kind("feed_forward", "gated", [](const PartSpec& s, BuildEnv& e) { return std::make_shared<GatedSiLU>(s, e, true); });
         register_latent_parts();
         register_moe_parts();
+        register_stream_parts();
         register_kind("block", "pre_norm", [](const PartSpec& s, BuildEnv& e) { return std::make_shared<PreNormBlock>(s, e); });
     });
 }

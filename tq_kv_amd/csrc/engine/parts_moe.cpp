@@ -11,8 +11,13 @@
 // over tiles of rows that belong to one expert, from lists that stay on the device, so the
 // launches are the same whatever the router chose and a step can be captured as a graph.
 //
-// params: hidden, inter, n_experts, top, router_scale, gate / limit / alpha, shared (a feed-forward
-// part spec, or null); optional names {router, expert (with %d for the expert's number), gate, up,
+// Variants, all parameters: gated false makes an expert down(f(up_proj x)), f the gate's function of one product
+// (relu2: max(z, 0)^2), without a gate product and its tensor; normalize "chosen" makes the weights the softmax over
+// the chosen logits alone (times router_scale); shared_gate names a tensor [1, hidden] whose product with x, through
+// a sigmoid, multiplies the shared expert's output token by token.
+//
+// params: hidden, inter, n_experts, top, router_scale, gate / limit / alpha, gated, normalize, shared (a feed-forward
+// part spec, or null), shared_gate (a tensor's name, or null); optional names {router, expert (with %d for the expert's number), gate, up,
 // down, shared}.  Tensors: router [experts, hidden]; per expert gate, up [inter, hidden], down
 // [hidden, inter]; the shared expert's own under its prefix.
 #include "kernels.h"
@@ -39,6 +44,11 @@ public:
         top_ = (int)r.integer("top", 1);
         router_scale_ = (float)r.number_or("router_scale", 1.0);
         gate_ = Gate::from_params(r, "routed_experts");
+        gated_ = r.boolean_or("gated", true);
+        const std::string normalize = r.string_or("normalize", "all");
+        if (normalize != "all" && normalize != "chosen") raise(TQE_ERR_ARGUMENT, "routed_experts: unknown normalize '%s' (known: all, chosen)", normalize.c_str());
+        renormalize_ = normalize == "chosen";
+        n_shared_gate_ = r.string_or("shared_gate", "");
         if (top_ > n_experts_) raise(TQE_ERR_ARGUMENT, "routed_experts: top %d of %d experts", top_, n_experts_);
         const int most = K::moe_max_experts.raw();
         if (n_experts_ > most) raise(TQE_ERR_CONFIG, "routed_experts: %d experts are more than the kernels take (%d)", n_experts_, most);
@@ -58,6 +68,7 @@ public:
             if (!shared_) raise(TQE_ERR_ARGUMENT, "routed_experts: the shared expert is no feed-forward");
             graph_safe = shared_->graph_safe;
         }
+        if (!n_shared_gate_.empty() && !shared_) raise(TQE_ERR_ARGUMENT, "routed_experts: a gate for a shared expert that is not there");
     }
 
     std::string expert_prefix(int e) const {
@@ -70,12 +81,13 @@ public:
         TensorSpecs t = {{n_router_, w(n_experts_, hidden_)}};
         for (int e = 0; e < n_experts_; ++e) {
             const std::string p = expert_prefix(e);
-            t.push_back({p + n_gate_, w(inter_, hidden_)});
+            if (gated_) t.push_back({p + n_gate_, w(inter_, hidden_)});
             t.push_back({p + n_up_, w(inter_, hidden_)});
             t.push_back({p + n_down_, w(hidden_, inter_)});
         }
         if (shared_)
             for (const auto& s : shared_->tensors()) t.push_back({n_shared_ + s.first, s.second});
+        if (!n_shared_gate_.empty()) t.push_back({n_shared_gate_, w(1, hidden_)});
         return t;
     }
     void load(Loaded& t, hipStream_t stream) override {
@@ -84,7 +96,7 @@ public:
         std::vector<OwnedPtr> gu, down;
         for (int e = 0; e < n_experts_; ++e) {
             const std::string p = expert_prefix(e);
-            gu.push_back(take(t, p + n_gate_));
+            if (gated_) gu.push_back(take(t, p + n_gate_));
             gu.push_back(take(t, p + n_up_));
             down.push_back(take(t, p + n_down_));
         }
@@ -95,9 +107,11 @@ public:
             for (const auto& s : shared_->tensors()) own[s.first] = take(t, n_shared_ + s.first);
             shared_->load(own, stream);
         }
+        if (!n_shared_gate_.empty()) shared_gate_ = take(t, n_shared_gate_);
     }
     OwnedPtr held(const std::string& name) const override {
         if (name == n_router_) return router_;
+        if (!n_shared_gate_.empty() && name == n_shared_gate_) return shared_gate_;
         if (name == "experts.gate_up") return gate_up_;
         if (name == "experts.down") return down_;
         if (shared_ && name.compare(0, n_shared_.size(), n_shared_) == 0) return shared_->held(name.substr(n_shared_.size()));
@@ -125,29 +139,38 @@ public:
         int32_t* tile_expert = (int32_t*)tiles.data;
         int32_t* tile_row0 = tile_expert + max_tiles;
         int32_t* tile_rows = tile_row0 + max_tiles;
-        K::moe_route(x.x.data, dtype, router_->t.data, router_->t.dtype, n_experts_, (int)hidden_, top_, router_scale_, (int32_t*)idx.data,
+        K::moe_route(x.x.data, dtype, router_->t.data, router_->t.dtype, n_experts_, (int)hidden_, top_, router_scale_, renormalize_ ? 1 : 0, (int32_t*)idx.data,
                      (float*)weight.data, (int)n, c.stream);
         K::moe_group((const int32_t*)idx.data, (int)n, top_, n_experts_, tile_m, (int32_t*)pair_pos.data, (int32_t*)sorted_tok.data, tile_expert, tile_row0,
                      tile_rows, (int32_t*)n_tiles.data, c.stream);
         Tensor shared_out;
         if (shared_) shared_out = shared_->forward(c, x, nullptr);
+        Tensor shared_scale;
+        if (shared_gate_) {
+            shared_scale = c.alloc(F32, {n});
+            K::row_gate(x.x.data, dtype, shared_gate_->t.data, shared_gate_->t.dtype, (float*)shared_scale.data, (int)n, (int)hidden_, c.stream);
+        }
+        // an expert's first product: gate and up side by side, or up alone with the gate's function of it
+        const int first = gated_ ? 1 : 2;
+        const long long first_stride = (long long)(gated_ ? 2 : 1) * inter_ * hidden_;
         Tensor act = c.alloc(dtype, {pairs, inter_});
         Tensor y = c.alloc(dtype, {pairs, hidden_});
         if (on_cores) {
-            K::moe_product_mfma(x.x.data, (const int32_t*)sorted_tok.data, gate_up_->t.data, (long long)(2 * inter_ * hidden_), act.data, (int)inter_,
-                                (int)hidden_, 1, gate_.kind, gate_.limit, gate_.alpha, tile_expert, tile_row0, tile_rows,
+            K::moe_product_mfma(x.x.data, (const int32_t*)sorted_tok.data, gate_up_->t.data, first_stride, act.data, (int)inter_,
+                                (int)hidden_, first, gate_.kind, gate_.limit, gate_.alpha, tile_expert, tile_row0, tile_rows,
                                 (const int32_t*)n_tiles.data, max_tiles, tile_m, c.stream);
             K::moe_product_mfma(act.data, nullptr, down_->t.data, (long long)(hidden_ * inter_), y.data, (int)hidden_, (int)inter_, 0, 0, 0.f, 1.f,
                                 tile_expert, tile_row0, tile_rows, (const int32_t*)n_tiles.data, max_tiles, tile_m, c.stream);
         } else {
-            K::moe_product(x.x.data, dtype, (const int32_t*)sorted_tok.data, gate_up_->t.data, gate_up_->t.dtype, (long long)(2 * inter_ * hidden_),
-                           act.data, (int)inter_, (int)hidden_, 1, gate_.kind, gate_.limit, gate_.alpha, tile_expert, tile_row0, tile_rows,
+            K::moe_product(x.x.data, dtype, (const int32_t*)sorted_tok.data, gate_up_->t.data, gate_up_->t.dtype, first_stride,
+                           act.data, (int)inter_, (int)hidden_, first, gate_.kind, gate_.limit, gate_.alpha, tile_expert, tile_row0, tile_rows,
                            (const int32_t*)n_tiles.data, max_tiles, c.stream);
             K::moe_product(act.data, dtype, nullptr, down_->t.data, down_->t.dtype, (long long)(hidden_ * inter_), y.data, (int)hidden_, (int)inter_, 0,
                            0, 0.f, 1.f, tile_expert, tile_row0, tile_rows, (const int32_t*)n_tiles.data, max_tiles, c.stream);
         }
         Tensor out = c.alloc(dtype, {n, hidden_});
-        K::moe_combine(y.data, dtype, (const int32_t*)pair_pos.data, (const float*)weight.data, top_, shared_out.data, out.data, (int)n,
+        K::moe_combine(y.data, dtype, (const int32_t*)pair_pos.data, (const float*)weight.data, top_, shared_out.data,
+                       shared_gate_ ? (const float*)shared_scale.data : nullptr, out.data, (int)n,
                        (int)hidden_, c.stream);
         return out;
     }
@@ -157,6 +180,9 @@ private:
     int n_experts_, top_;
     float router_scale_;
     Gate gate_;
+    bool gated_ = true, renormalize_ = false;
+    std::string n_shared_gate_;
+    OwnedPtr shared_gate_;
     std::string n_router_, n_expert_, n_gate_, n_up_, n_down_, n_shared_;
     std::shared_ptr<FeedForward> shared_;
     OwnedPtr router_, gate_up_, down_;

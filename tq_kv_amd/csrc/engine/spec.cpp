@@ -63,6 +63,7 @@ Json CacheNeed::to_json() const {
         j.set("key_page", shape_json(key_page));
         j.set("value_page", shape_json(value_page));
         j.set("window", window > 0 ? Json(window) : Json());
+        if (keep_first > 0) j.set("keep_first", keep_first);
     } else {
         j.set("kind", "state");
         j.set("shape", shape_json(state_shape));
@@ -81,6 +82,8 @@ CacheNeed CacheNeed::from_json(const Json& j) {
         n.value_page = shape_from(j["value_page"], "cache need");
         if (j["window"].is_int()) n.window = (int)j["window"].as_int();
         if (n.window < 0) raise(TQE_ERR_ARGUMENT, "cache need: window %d", n.window);
+        if (j["keep_first"].is_int()) n.keep_first = (int)j["keep_first"].as_int();
+        if (n.keep_first < 0) raise(TQE_ERR_ARGUMENT, "cache need: keep_first %d", n.keep_first);
     } else if (kind == "state") {
         n.kind = State;
         n.state_shape = shape_from(j["shape"], "cache need");

@@ -41,17 +41,18 @@ struct PartSpec {
 
 // What a mixer keeps per sequence.  Pages: keys and values for every position, in pages of
 // TQE_PAGE positions whose layout is the mixer's own: key_page and value_page are the shapes
-// of one page (window > 0: only the last `window` positions are ever read).  State: a
+// of one page (window > 0: only the last `window` positions are ever read, and the first `keep_first`).  State: a
 // fixed-size row per sequence, zero at the start.
 struct CacheNeed {
     enum Kind { None = 0, Pages = 1, State = 2 };
     int kind = None;
     std::vector<int64_t> key_page, value_page;
     int window = 0;
+    int keep_first = 0;          // with a window: the sequence's first positions that stay visible whatever the window
     std::vector<int64_t> state_shape;
     int state_dtype = F32;
     bool operator==(const CacheNeed& o) const {
-        return kind == o.kind && key_page == o.key_page && value_page == o.value_page && window == o.window &&
+        return kind == o.kind && key_page == o.key_page && value_page == o.value_page && window == o.window && keep_first == o.keep_first &&
                state_shape == o.state_shape && state_dtype == o.state_dtype;
     }
     Json to_json() const;

@@ -52,6 +52,7 @@ void StepContext::plan(const tqe_cache* cache, int n, const int32_t* slots, cons
     }
     tiles_.clear();
     memo.clear();
+    carried.clear();
 }
 
 void StepContext::upload(int32_t* into) {

@@ -90,6 +90,7 @@ struct StepContext {
     // scratch of the model for a step whose last block goes on with a few rows
     std::unique_ptr<struct Stream> sub_stream;
     std::map<std::string, int> memo;                 // what parts remember for the length of a step (the prompt kernel's tile)
+    std::map<std::string, Tensor> carried;           // what a part hands to later parts of the same step (memory of the step's arena)
 
     StepContext();
     ~StepContext();

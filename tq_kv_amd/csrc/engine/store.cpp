@@ -61,6 +61,8 @@ CacheStore::CacheStore(const std::vector<CacheNeed>& needs, const std::vector<in
     for (const PageGroup& g : page_groups) { pages.push_back(g.n_pages); windows.push_back(g.need.window); }
     book = tqe_cache_new(max_slots, (int)page_groups.size(), pages.data(), windows.data());
     if (!book) throw Error(TQE_ERR_ARGUMENT, tqe_last_error());
+    for (size_t g = 0; g < page_groups.size(); ++g)
+        if (page_groups[g].need.keep_first > 0) check_status(tqe_cache_keep_first(book, (int)g, page_groups[g].need.keep_first));
 
     // what each run sees
     entries_.assign(n_runs, CacheEntry());
@@ -87,6 +89,7 @@ CacheStore::CacheStore(const std::vector<CacheNeed>& needs, const std::vector<in
             const PageGroup& g = page_groups[p.group];
             e.group = (int)p.group;
             e.window = need.window;
+            e.keep_first = need.keep_first;
             e.keys = g.keys->t.slice(p.index, p.index + 1);
             e.values = g.values->t.slice(p.index, p.index + 1);
             // drop the leading dimension of one run

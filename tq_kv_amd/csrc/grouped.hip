@@ -43,6 +43,7 @@ struct GroupedArgs {
     int N, K;
     int gate;
     float gate_limit, gate_alpha;
+    int activated;                  // not gated: the gate's function of the product itself is applied (see act_value)
     // tiles from lists on the device (tile_group != null), or every group over all rows in tiles of tile_rows_max
     const int32_t *tile_group, *tile_row0, *tile_rows, *n_tiles;
     int n_groups, n_rows, tile_rows_max;
@@ -206,6 +207,8 @@ void grouped_mfma_kernel(GroupedArgs p) {
                     // gate and up rounded as stored products would be, then the gate in float32
                     const float gv = to_float(from_float<bf16_t>(v)), uv = to_float(from_float<bf16_t>(acc[NB - 1][rt][cb][i]));
                     v = gate_value(p.gate, p.gate_limit, p.gate_alpha, gv, uv);
+                } else if (p.activated) {
+                    v = act_value(p.gate, p.gate_limit, p.gate_alpha, to_float(from_float<bf16_t>(v)));
                 }
                 v *= scale;
                 const long long at = row * p.y_row_stride + (long long)group * p.y_group_stride + n;
@@ -241,17 +244,18 @@ extern "C" int tqk_moe_product_mfma(const void* x, const int32_t* x_rows, const 
     TQK_REQUIRE(x && w && y && tile_expert && tile_row0 && tile_rows && n_tiles, "tqk_moe_product_mfma: null pointer");
     TQK_REQUIRE(N > 0 && K > 0 && K % 8 == 0 && max_tiles >= 0 && max_tiles <= 65535, "tqk_moe_product_mfma: bad sizes (N %d, K %d, %d tiles)", N, K, max_tiles);
     TQK_REQUIRE(tile_m == 16 || tile_m == 32 || tile_m == 64, "tqk_moe_product_mfma: tiles of %d rows", tile_m);
+    TQK_REQUIRE(gated >= 0 && gated <= 2, "tqk_moe_product_mfma: gated must be 0, 1 or 2, got %d", gated);
     TQK_REQUIRE(!gated || (gate >= 0 && gate < TQK_GATE_KINDS), "tqk_moe_product_mfma: unknown gate %d", gate);
-    TQK_REQUIRE(expert_stride >= (long long)(gated ? 2 : 1) * N * K && expert_stride % 8 == 0, "tqk_moe_product_mfma: experts overlap or are not aligned");
+    TQK_REQUIRE(expert_stride >= (long long)(gated == 1 ? 2 : 1) * N * K && expert_stride % 8 == 0, "tqk_moe_product_mfma: experts overlap or are not aligned");
     TQK_REQUIRE(((((uintptr_t)x) | ((uintptr_t)w)) & 15) == 0, "tqk_moe_product_mfma: x and w must be 16-byte aligned");
     if (max_tiles == 0) return 0;
     GroupedArgs a = {};
     a.x = x; a.x_row_stride = K; a.x_rows = x_rows;
     a.w = (const bf16_t*)w; a.w_group_stride = expert_stride;
     a.y = y; a.y_row_stride = N;
-    a.N = N; a.K = K; a.gate = gate; a.gate_limit = limit; a.gate_alpha = alpha;
+    a.N = N; a.K = K; a.gate = gate; a.gate_limit = limit; a.gate_alpha = alpha; a.activated = gated == 2;
     a.tile_group = tile_expert; a.tile_row0 = tile_row0; a.tile_rows = tile_rows; a.n_tiles = n_tiles; a.tile_rows_max = tile_m;
-    return gated ? launch_grouped<true>(a, max_tiles, (hipStream_t)stream) : launch_grouped<false>(a, max_tiles, (hipStream_t)stream);
+    return gated == 1 ? launch_grouped<true>(a, max_tiles, (hipStream_t)stream) : launch_grouped<false>(a, max_tiles, (hipStream_t)stream);
 }
 
 /* y[t, h, :N] = scale[t, h] * W_h x[t, h, :K] for every token t and head h.  x: [tokens, heads, x_head_stride...] rows of

@@ -161,6 +161,7 @@ struct PagePool {
 struct Group {
     PagePool pool;
     int window = 0;                                   // 0: every position stays
+    int keep_first = 0;                               // with a window: pages that hold any of the first keep_first positions stay too
     std::vector<std::vector<int32_t>> pages;          // per slot: page of positions 64 i .. , -1 where given back
     std::vector<uint8_t> known;                       // per slot: whether the slot has a list at all
 };
@@ -223,6 +224,13 @@ tqe_cache_t* tqe_cache_new(int max_slots, int n_groups, const int32_t* pages_per
 }
 
 void tqe_cache_free(tqe_cache_t* c) { delete c; }
+
+int tqe_cache_keep_first(tqe_cache_t* c, int group, int positions) {
+    if (!c || group < 0 || group >= (int)c->groups.size() || positions < 0)
+        return fail(TQE_ERR_ARGUMENT, "tqe_cache_keep_first: group %d, %d positions", group, positions);
+    c->groups[group].keep_first = positions;
+    return TQE_OK;
+}
 
 int tqe_cache_acquire(tqe_cache_t* c, int32_t* slot_out) try {
     if (!c || !slot_out) return fail(TQE_ERR_ARGUMENT, "tqe_cache_acquire: null pointer");
@@ -325,7 +333,7 @@ int tqe_cache_commit(tqe_cache_t* c, int n, const int32_t* slots, const int32_t*
             std::vector<int32_t>& have = g.pages[s];
             const int first_needed = std::max(0, c->lengths[s] + 1 - g.window);
             const int dead = std::min(first_needed / TQE_PAGE, (int)have.size());
-            for (int k = 0; k < dead; ++k)
+            for (int k = pages_for(g.keep_first); k < dead; ++k)
                 if (have[k] >= 0) { g.pool.give_back(have[k]); have[k] = -1; }
         }
     }

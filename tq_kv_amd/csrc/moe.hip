@@ -26,7 +26,7 @@
 // under way at once, added up in a fixed order), then the first wave takes the softmax and the largest.
 template <typename TA, typename TW>
 __global__ __launch_bounds__(MOE_ROUTE_WAVES * TQK_WAVE)
-void moe_route_kernel(const TA* __restrict__ x, const TW* __restrict__ w, int n_experts, int hidden, int top, float scale,
+void moe_route_kernel(const TA* __restrict__ x, const TW* __restrict__ w, int n_experts, int hidden, int top, float scale, int renormalize,
                       int32_t* __restrict__ idx, float* __restrict__ weight) {
     __shared__ float z[MOE_MAX_EXPERTS];
     const int wave = threadIdx.x / TQK_WAVE, lane = threadIdx.x % TQK_WAVE;
@@ -90,6 +90,13 @@ void moe_route_kernel(const TA* __restrict__ x, const TW* __restrict__ w, int n_
             idx[(size_t)t * top + k] = best_e;
             weight[(size_t)t * top + k] = expf(best - m) / sum * scale;
         }
+    }
+    if (!renormalize) return;
+    // the softmax over the chosen logits alone: the chosen scores divided by their sum, added up in the order they were chosen
+    if (lane == 0) {
+        float chosen = 0.f;
+        for (int k = 0; k < top; ++k) chosen += weight[(size_t)t * top + k];
+        for (int k = 0; k < top; ++k) weight[(size_t)t * top + k] /= chosen;
     }
 }
 
@@ -197,6 +204,8 @@ void moe_product_kernel(const TX* __restrict__ x, const int32_t* __restrict__ x_
                 // gate and up are rounded as stored products would be, then the gate in float32
                 const float g = to_float(from_float<TY>(v)), u = to_float(from_float<TY>(acc[GATED ? 1 : 0][i][j]));
                 v = gate_value(gate, limit, alpha, g, u);
+            } else if (gate >= 0) {
+                v = act_value(gate, limit, alpha, to_float(from_float<TY>(v)));
             }
             y[(size_t)(row0 + r) * N + n] = from_float<TY>(v);
         }
@@ -207,7 +216,7 @@ void moe_product_kernel(const TX* __restrict__ x, const int32_t* __restrict__ x_
 template <typename TA>
 __global__ __launch_bounds__(256)
 void moe_combine_kernel(const TA* __restrict__ y, const int32_t* __restrict__ pair_pos, const float* __restrict__ weight, int top,
-                        const TA* __restrict__ shared, TA* __restrict__ out, int hidden) {
+                        const TA* __restrict__ shared, const float* __restrict__ shared_scale, TA* __restrict__ out, int hidden) {
     // the token's rows and weights once, side by side, not one load after the other in front of every element
     __shared__ int32_t row[MOE_MAX_EXPERTS];
     __shared__ float wt[MOE_MAX_EXPERTS];
@@ -217,11 +226,12 @@ void moe_combine_kernel(const TA* __restrict__ y, const int32_t* __restrict__ pa
         wt[k] = weight[(size_t)t * top + k];
     }
     __syncthreads();
+    const float ss = shared && shared_scale ? shared_scale[t] : 1.f;
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
         float v = 0.f;
 #pragma unroll 4
         for (int k = 0; k < top; ++k) v = fmaf(wt[k], to_float(y[(size_t)row[k] * hidden + i]), v);
-        if (shared) v += to_float(shared[(size_t)t * hidden + i]);
+        if (shared) v = fmaf(ss, to_float(shared[(size_t)t * hidden + i]), v);
         out[(size_t)t * hidden + i] = from_float<TA>(v);
     }
 }
@@ -232,14 +242,14 @@ extern "C" int tqk_moe_tile_rows(void) { return MOE_TM; }
 extern "C" int tqk_moe_max_tiles(int n_pairs, int n_experts, int tile_m) { return (n_pairs + tile_m - 1) / tile_m + n_experts; }
 
 extern "C" int tqk_moe_route(const void* x, int act_dtype, const void* w_router, int w_dtype, int n_experts, int hidden, int top, float scale,
-                             int32_t* idx, float* weight, int n_tokens, void* stream) {
+                             int renormalize, int32_t* idx, float* weight, int n_tokens, void* stream) {
     TQK_REQUIRE(x && w_router && idx && weight, "tqk_moe_route: null pointer");
     TQK_REQUIRE(n_experts > 0 && n_experts <= MOE_MAX_EXPERTS, "tqk_moe_route: %d experts, the kernel takes 1 to %d", n_experts, MOE_MAX_EXPERTS);
     TQK_REQUIRE(top > 0 && top <= n_experts && hidden > 0 && n_tokens >= 0, "tqk_moe_route: bad sizes (top %d of %d experts)", top, n_experts);
     if (n_tokens == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
 #define TQK_ROUTE(TA, TW) \
-    moe_route_kernel<TA, TW><<<n_tokens, MOE_ROUTE_WAVES * TQK_WAVE, 0, s>>>((const TA*)x, (const TW*)w_router, n_experts, hidden, top, scale, idx, weight)
+    moe_route_kernel<TA, TW><<<n_tokens, MOE_ROUTE_WAVES * TQK_WAVE, 0, s>>>((const TA*)x, (const TW*)w_router, n_experts, hidden, top, scale, renormalize, idx, weight)
     if (act_dtype == TQK_F32 && w_dtype == TQK_F32) TQK_ROUTE(float, float);
     else if (act_dtype == TQK_F32 && w_dtype == TQK_BF16) TQK_ROUTE(float, bf16_t);
     else if (act_dtype == TQK_BF16 && w_dtype == TQK_F32) TQK_ROUTE(bf16_t, float);
@@ -266,11 +276,11 @@ static int launch_moe_product(const void* x, const int32_t* x_rows, const void* 
                               int gate, float limit, float alpha, const int32_t* tile_expert, const int32_t* tile_row0,
                               const int32_t* tile_rows, const int32_t* n_tiles, int max_tiles, hipStream_t s) {
     dim3 grid((N + MOE_TN - 1) / MOE_TN, max_tiles);
-    if (gated)
+    if (gated == 1)
         moe_product_kernel<TX, TW, TY, true><<<grid, 256, 0, s>>>((const TX*)x, x_rows, (const TW*)w, expert_stride, (TY*)y, N, K, gate, limit, alpha,
                                                                   tile_expert, tile_row0, tile_rows, n_tiles);
     else
-        moe_product_kernel<TX, TW, TY, false><<<grid, 256, 0, s>>>((const TX*)x, x_rows, (const TW*)w, expert_stride, (TY*)y, N, K, gate, limit, alpha,
+        moe_product_kernel<TX, TW, TY, false><<<grid, 256, 0, s>>>((const TX*)x, x_rows, (const TW*)w, expert_stride, (TY*)y, N, K, gated == 2 ? gate : -1, limit, alpha,
                                                                    tile_expert, tile_row0, tile_rows, n_tiles);
     return tqk_check_launch("tqk_moe_product");
 }
@@ -280,8 +290,9 @@ extern "C" int tqk_moe_product(const void* x, int act_dtype, const int32_t* x_ro
                                const int32_t* tile_row0, const int32_t* tile_rows, const int32_t* n_tiles, int max_tiles, void* stream) {
     TQK_REQUIRE(x && w && y && tile_expert && tile_row0 && tile_rows && n_tiles, "tqk_moe_product: null pointer");
     TQK_REQUIRE(N > 0 && K > 0 && max_tiles >= 0 && max_tiles <= 65535, "tqk_moe_product: bad sizes (N %d, K %d, %d tiles)", N, K, max_tiles);
+    TQK_REQUIRE(gated >= 0 && gated <= 2, "tqk_moe_product: gated must be 0 (plain), 1 (gate and up) or 2 (one product with its activation), got %d", gated);
     TQK_REQUIRE(!gated || (gate >= 0 && gate < TQK_GATE_KINDS), "tqk_moe_product: unknown gate %d", gate);
-    TQK_REQUIRE(expert_stride >= (long long)(gated ? 2 : 1) * N * K, "tqk_moe_product: experts overlap");
+    TQK_REQUIRE(expert_stride >= (long long)(gated == 1 ? 2 : 1) * N * K, "tqk_moe_product: experts overlap");
     /* the tile lists must have been made for tiles of tqk_moe_tile_rows() rows */
     if (max_tiles == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
@@ -295,16 +306,16 @@ extern "C" int tqk_moe_product(const void* x, int act_dtype, const int32_t* x_ro
     return tqk_fail("tqk_moe_product: unknown dtypes %d, %d", act_dtype, w_dtype);
 }
 
-extern "C" int tqk_moe_combine(const void* y, int act_dtype, const int32_t* pair_pos, const float* weight, int top, const void* shared, void* out,
-                               int n_tokens, int hidden, void* stream) {
+extern "C" int tqk_moe_combine(const void* y, int act_dtype, const int32_t* pair_pos, const float* weight, int top, const void* shared,
+                               const float* shared_scale, void* out, int n_tokens, int hidden, void* stream) {
     TQK_REQUIRE(y && pair_pos && weight && out, "tqk_moe_combine: null pointer");
     TQK_REQUIRE(top > 0 && top <= MOE_MAX_EXPERTS && hidden > 0 && n_tokens >= 0, "tqk_moe_combine: bad sizes");
     if (n_tokens == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     if (act_dtype == TQK_F32)
-        moe_combine_kernel<float><<<n_tokens, 256, 0, s>>>((const float*)y, pair_pos, weight, top, (const float*)shared, (float*)out, hidden);
+        moe_combine_kernel<float><<<n_tokens, 256, 0, s>>>((const float*)y, pair_pos, weight, top, (const float*)shared, shared_scale, (float*)out, hidden);
     else if (act_dtype == TQK_BF16)
-        moe_combine_kernel<bf16_t><<<n_tokens, 256, 0, s>>>((const bf16_t*)y, pair_pos, weight, top, (const bf16_t*)shared, (bf16_t*)out, hidden);
+        moe_combine_kernel<bf16_t><<<n_tokens, 256, 0, s>>>((const bf16_t*)y, pair_pos, weight, top, (const bf16_t*)shared, shared_scale, (bf16_t*)out, hidden);
     else return tqk_fail("tqk_moe_combine: unknown dtype %d", act_dtype);
     return tqk_check_launch("tqk_moe_combine");
 }

@@ -1,0 +1,150 @@
+// Small kernels on the residual stream and beside it: an embedding of hashed token pairs with
+// the previous token kept per sequence, a norm on a part's output that is added to the stream,
+// an activation of one product, and a per-token sigmoid gate.  float32 arithmetic throughout.
+#include "common.h"
+#include "tq_kernels.h"
+
+// ---- hashed pairs ------------------------------------------------------------------------------
+// h[t] += table[row], row = (prev * mul_prev + token * mul_cur) mod buckets, and the table's row
+// `buckets` for a sequence's first token.  The previous token is the one before it in the step, or,
+// for the first token a step brings of a sequence that has begun, what `last` holds for its slot.
+template <typename TT>
+__global__ __launch_bounds__(256)
+void pair_embed_kernel(const TT* __restrict__ table, int buckets, long long mul_prev, long long mul_cur, const int32_t* __restrict__ tokens,
+                       const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ seq_slot,
+                       const int32_t* __restrict__ seq_start, const int32_t* __restrict__ last, float* __restrict__ h, int hidden, int vocab) {
+    const int t = blockIdx.x;
+    const int pos = tok_pos[t], seq = tok_seq[t];
+    const int tok = tokens[t];
+    if (tok < 0 || tok >= vocab) return;
+    long long row = buckets;
+    if (pos > 0) {
+        const long long prev = pos > seq_start[seq] ? tokens[t - 1] : last[seq_slot[seq]];
+        row = (prev * mul_prev + (long long)tok * mul_cur) % buckets;
+        if (row < 0) row += buckets;
+    }
+    const TT* src = table + (size_t)row * hidden;
+    float* dst = h + (size_t)t * hidden;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] += to_float(src[i]);
+}
+
+// last[slot of sequence s] = the last token the step brings of s
+__global__ void remember_tokens_kernel(const int32_t* __restrict__ tokens, const int32_t* __restrict__ cu, const int32_t* __restrict__ seq_new,
+                                       const int32_t* __restrict__ seq_slot, int32_t* __restrict__ last, int n_seqs) {
+    const int s = blockIdx.x * blockDim.x + threadIdx.x;
+    if (s >= n_seqs || seq_new[s] <= 0) return;
+    last[seq_slot[s]] = tokens[cu[s] + seq_new[s] - 1];
+}
+
+// ---- norm of an output, added to the stream ------------------------------------------------------
+// h[t] += y[t] / sqrt(mean(y[t]^2) + eps) * w (w null: h[t] += y[t]); copy[t] = h[t] in the activation type.
+template <typename TA, typename TW>
+__global__ __launch_bounds__(256)
+void norm_add_kernel(float* __restrict__ h, const TA* __restrict__ y, const TW* __restrict__ w, float eps, TA* __restrict__ copy, int hidden) {
+    __shared__ float scratch[4];
+    const int t = blockIdx.x;
+    const TA* yr = y ? y + (size_t)t * hidden : nullptr;
+    float* hr = h + (size_t)t * hidden;
+    float inv = 1.f;
+    if (yr && w) {
+        float ss = 0.f;
+        for (int i = threadIdx.x; i < hidden; i += blockDim.x) { const float v = to_float(yr[i]); ss = fmaf(v, v, ss); }
+        ss = block_sum(ss, scratch);
+        inv = 1.f / sqrtf(ss / (float)hidden + eps);
+    }
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        float v = hr[i];
+        if (yr) {
+            v += w ? to_float(yr[i]) * inv * to_float(w[i]) : to_float(yr[i]);
+            hr[i] = v;
+        }
+        if (copy) copy[(size_t)t * hidden + i] = from_float<TA>(v);
+    }
+}
+
+template <typename TA>
+__global__ void unary_act_kernel(const TA* __restrict__ x, TA* __restrict__ out, long long n, int kind, float limit, float alpha) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = from_float<TA>(act_value(kind, limit, alpha, to_float(x[i])));
+}
+
+// out[t] = sigmoid(x[t] . w), a wave per token
+template <typename TA, typename TW>
+__global__ __launch_bounds__(256)
+void row_gate_kernel(const TA* __restrict__ x, const TW* __restrict__ w, float* __restrict__ out, int n_tokens, int hidden) {
+    const int t = blockIdx.x * 4 + threadIdx.x / TQK_WAVE, lane = threadIdx.x % TQK_WAVE;
+    if (t >= n_tokens) return;
+    const TA* xr = x + (size_t)t * hidden;
+    float d = 0.f;
+    for (int i = lane; i < hidden; i += TQK_WAVE) d = fmaf(to_float(xr[i]), to_float(w[i]), d);
+    d = wave_sum(d);
+    if (lane == 0) out[t] = 1.f / (1.f + expf(-d));
+}
+
+extern "C" int tqk_pair_embed(const void* table, int table_dtype, int buckets, long long mul_prev, long long mul_cur, const int32_t* tokens,
+                              const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* seq_slot, const int32_t* seq_start,
+                              const int32_t* last, float* h, int n_tokens, int hidden, int vocab, void* stream) {
+    TQK_REQUIRE(table && tokens && tok_seq && tok_pos && seq_slot && seq_start && last && h, "tqk_pair_embed: null pointer");
+    TQK_REQUIRE(buckets > 0 && hidden > 0 && n_tokens >= 0 && vocab > 0, "tqk_pair_embed: bad sizes");
+    TQK_REQUIRE(mul_prev >= 0 && mul_cur >= 0 && mul_prev < (1LL << 31) && mul_cur < (1LL << 31), "tqk_pair_embed: multipliers out of range");
+    if (n_tokens == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    if (table_dtype == TQK_F32)
+        pair_embed_kernel<float><<<n_tokens, 256, 0, s>>>((const float*)table, buckets, mul_prev, mul_cur, tokens, tok_seq, tok_pos, seq_slot, seq_start, last, h, hidden, vocab);
+    else if (table_dtype == TQK_BF16)
+        pair_embed_kernel<bf16_t><<<n_tokens, 256, 0, s>>>((const bf16_t*)table, buckets, mul_prev, mul_cur, tokens, tok_seq, tok_pos, seq_slot, seq_start, last, h, hidden, vocab);
+    else return tqk_fail("tqk_pair_embed: unknown dtype %d", table_dtype);
+    return tqk_check_launch("tqk_pair_embed");
+}
+
+extern "C" int tqk_remember_tokens(const int32_t* tokens, const int32_t* cu, const int32_t* seq_new, const int32_t* seq_slot, int32_t* last,
+                                   int n_seqs, void* stream) {
+    TQK_REQUIRE(tokens && cu && seq_new && seq_slot && last, "tqk_remember_tokens: null pointer");
+    if (n_seqs <= 0) return 0;
+    remember_tokens_kernel<<<(n_seqs + 255) / 256, 256, 0, (hipStream_t)stream>>>(tokens, cu, seq_new, seq_slot, last, n_seqs);
+    return tqk_check_launch("tqk_remember_tokens");
+}
+
+extern "C" int tqk_norm_add(float* h, const void* y, int act_dtype, const void* weight, int weight_dtype, float eps, void* copy, int n_tokens,
+                            int hidden, void* stream) {
+    TQK_REQUIRE(h && (y || copy), "tqk_norm_add: null pointer");
+    TQK_REQUIRE(n_tokens >= 0 && hidden > 0, "tqk_norm_add: bad sizes");
+    if (n_tokens == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+#define TQK_NA(TA, TW) norm_add_kernel<TA, TW><<<n_tokens, 256, 0, s>>>(h, (const TA*)y, (const TW*)weight, eps, (TA*)copy, hidden)
+    if (act_dtype == TQK_F32 && weight_dtype == TQK_F32) TQK_NA(float, float);
+    else if (act_dtype == TQK_F32 && weight_dtype == TQK_BF16) TQK_NA(float, bf16_t);
+    else if (act_dtype == TQK_BF16 && weight_dtype == TQK_F32) TQK_NA(bf16_t, float);
+    else if (act_dtype == TQK_BF16 && weight_dtype == TQK_BF16) TQK_NA(bf16_t, bf16_t);
+    else return tqk_fail("tqk_norm_add: unknown dtypes %d, %d", act_dtype, weight_dtype);
+#undef TQK_NA
+    return tqk_check_launch("tqk_norm_add");
+}
+
+extern "C" int tqk_unary_act(const void* x, void* out, int act_dtype, long long n, int kind, float limit, float alpha, void* stream) {
+    TQK_REQUIRE(x && out && n >= 0, "tqk_unary_act: null pointer");
+    TQK_REQUIRE(kind >= 0 && kind < TQK_GATE_KINDS, "tqk_unary_act: unknown activation %d", kind);
+    if (n == 0) return 0;
+    const long long blocks = (n + 255) / 256;
+    TQK_REQUIRE(blocks <= 0x7fffffff, "tqk_unary_act: too many elements");
+    hipStream_t s = (hipStream_t)stream;
+    if (act_dtype == TQK_F32) unary_act_kernel<float><<<(unsigned)blocks, 256, 0, s>>>((const float*)x, (float*)out, n, kind, limit, alpha);
+    else if (act_dtype == TQK_BF16) unary_act_kernel<bf16_t><<<(unsigned)blocks, 256, 0, s>>>((const bf16_t*)x, (bf16_t*)out, n, kind, limit, alpha);
+    else return tqk_fail("tqk_unary_act: unknown dtype %d", act_dtype);
+    return tqk_check_launch("tqk_unary_act");
+}
+
+extern "C" int tqk_row_gate(const void* x, int act_dtype, const void* w, int w_dtype, float* out, int n_tokens, int hidden, void* stream) {
+    TQK_REQUIRE(x && w && out, "tqk_row_gate: null pointer");
+    TQK_REQUIRE(n_tokens >= 0 && hidden > 0, "tqk_row_gate: bad sizes");
+    if (n_tokens == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+#define TQK_RG(TA, TW) row_gate_kernel<TA, TW><<<(n_tokens + 3) / 4, 256, 0, s>>>((const TA*)x, (const TW*)w, out, n_tokens, hidden)
+    if (act_dtype == TQK_F32 && w_dtype == TQK_F32) TQK_RG(float, float);
+    else if (act_dtype == TQK_F32 && w_dtype == TQK_BF16) TQK_RG(float, bf16_t);
+    else if (act_dtype == TQK_BF16 && w_dtype == TQK_F32) TQK_RG(bf16_t, float);
+    else if (act_dtype == TQK_BF16 && w_dtype == TQK_BF16) TQK_RG(bf16_t, bf16_t);
+    else return tqk_fail("tqk_row_gate: unknown dtypes %d, %d", act_dtype, w_dtype);
+#undef TQK_RG
+    return tqk_check_launch("tqk_row_gate");
+}

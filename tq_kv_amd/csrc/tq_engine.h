@@ -20,7 +20,7 @@ extern "C" {
 #endif
 
 #define TQE_PAGE 64             /* positions per cache page (the kernel library is asked for its own and must agree) */
-#define TQE_KERNEL_ABI 18       /* the version of the kernel library's interface (tqk_abi_version) this engine is written against */
+#define TQE_KERNEL_ABI 19       /* the version of the kernel library's interface (tqk_abi_version) this engine is written against */
 #define TQE_MAX_GROUPS 16       /* groups of cached runs a cache may have */
 
 enum {
@@ -58,6 +58,9 @@ typedef struct tqe_cache tqe_cache_t;
  * back than the window of the next query.  Returns NULL on error. */
 tqe_cache_t* tqe_cache_new(int max_slots, int n_groups, const int32_t* pages_per_group, const int32_t* window_per_group);
 void tqe_cache_free(tqe_cache_t* cache);
+/* A group with a window also keeps the pages that hold any of a sequence's first `positions` positions (set before the
+ * cache is used; 0, the default: the window alone decides). */
+int tqe_cache_keep_first(tqe_cache_t* cache, int group, int positions);
 
 /* A free slot with length 0 (TQE_ERR_FULL if there is none); everything a slot holds goes back. */
 int tqe_cache_acquire(tqe_cache_t* cache, int32_t* slot_out);

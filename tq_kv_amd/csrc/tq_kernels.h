@@ -176,7 +176,7 @@ int tqk_attention_prefill(const void* q, const void* keys, const void* values, c
 int tqk_swiglu(const void* gate_up, void* out, int act_dtype, int n_tokens, int inter, void* stream);
 
 /* Gates of feed-forwards other than SiLU.  gate: 0 g sigmoid(g) u; 1 max(g, 0) u; 2 g' sigmoid(alpha g') (u' + 1) with
- * g' = min(g, limit) and u' = clamp(u, -limit, limit); 3 gelu_tanh(g) u.  tqk_gated_act is tqk_swiglu, and
+ * g' = min(g, limit) and u' = clamp(u, -limit, limit); 3 gelu_tanh(g) u; 4 max(g, 0)^2 u.  tqk_gated_act is tqk_swiglu, and
  * tqk_fused_gated_act and tqk_mid_gated_act are tqk_fused_gated and tqk_mid_gated, with the gate named. */
 int tqk_gated_act(const void* gate_up, void* out, int act_dtype, int n_tokens, int inter, int gate, float limit, float alpha,
                   void* stream);
@@ -232,12 +232,15 @@ int tqk_latent_values(const float* o, const void* w_uv, int w_dtype, const float
  * among its expert's rows, sorted_tok[row] names the row's token; tile lists of tqk_moe_max_tiles(pairs, experts)
  * entries and their number *n_tiles, all on the device.  tqk_moe_product: rows (x[x_rows[row]] or x[row]) of every
  * tile times its expert's weight (w + expert * expert_stride: [N, K], gated: gate rows then up rows [2 N, K]) into
- * y [pairs, N].  tqk_moe_combine: out[t] = sum_k weight[t, k] y[pair_pos[t, k]] + shared[t] (shared may be null). */
+ * y [pairs, N]; gated 0: the product alone, 1: gate and up, 2: one product [N, K] with the gate's function of it alone (u = 1:
+ * relu2 gives max(z, 0)^2).  tqk_moe_route with renormalize: the chosen weights are divided by their sum (the softmax over
+ * the chosen logits alone).  tqk_moe_combine: out[t] = sum_k weight[t, k] y[pair_pos[t, k]] + shared_scale[t] * shared[t]
+ * (shared may be null; shared_scale null: 1). */
 int tqk_moe_max_experts(void);
 int tqk_moe_tile_rows(void);
 int tqk_moe_max_tiles(int n_pairs, int n_experts, int tile_m);
 int tqk_moe_route(const void* x, int act_dtype, const void* w_router, int w_dtype, int n_experts, int hidden, int top, float scale,
-                  int32_t* idx, float* weight, int n_tokens, void* stream);
+                  int renormalize, int32_t* idx, float* weight, int n_tokens, void* stream);
 int tqk_moe_group(const int32_t* idx, int n_tokens, int top, int n_experts, int tile_m, int32_t* pair_pos, int32_t* sorted_tok,
                   int32_t* tile_expert, int32_t* tile_row0, int32_t* tile_rows, int32_t* n_tiles, void* stream);
 int tqk_moe_product(const void* x, int act_dtype, const int32_t* x_rows, const void* w, int w_dtype, long long expert_stride, void* y,
@@ -254,8 +257,45 @@ int tqk_moe_product_mfma(const void* x, const int32_t* x_rows, const void* w, lo
 int tqk_head_product(const void* x, int x_f32, long long x_row_stride, long long x_head_stride, const void* w, void* y, int y_f32,
                      long long y_row_stride, long long y_head_stride, const float* scale, int n_tokens, int n_heads, int N, int K,
                      void* stream);
-int tqk_moe_combine(const void* y, int act_dtype, const int32_t* pair_pos, const float* weight, int top, const void* shared, void* out,
-                    int n_tokens, int hidden, void* stream);
+int tqk_moe_combine(const void* y, int act_dtype, const int32_t* pair_pos, const float* weight, int top, const void* shared,
+                    const float* shared_scale, void* out, int n_tokens, int hidden, void* stream);
+
+/* Around the residual stream (stream_ops.hip).  tqk_pair_embed: h[t] += table[(prev * mul_prev + token * mul_cur) mod buckets],
+ * table [buckets + 1, hidden], the last row for a sequence's first token; prev is the token before it in the step or, for the
+ * first token a step brings of a sequence that has begun, last[slot].  tqk_remember_tokens: last[slot] = the last token the step
+ * brings of each sequence (its own launch: the first token of a sequence's piece reads what the last one writes).
+ * tqk_norm_add: h[t] += y[t] / sqrt(mean(y[t]^2) + eps) * weight (weight null: h[t] += y[t]; y null: nothing is added), and
+ * copy[t] = h[t] in the activation type (copy may be null).  tqk_unary_act: out = f(x), f a gate's function with u = 1.
+ * tqk_row_gate: out[t] = sigmoid(x[t] . w), float32. */
+int tqk_pair_embed(const void* table, int table_dtype, int buckets, long long mul_prev, long long mul_cur, const int32_t* tokens,
+                   const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* seq_slot, const int32_t* seq_start,
+                   const int32_t* last, float* h, int n_tokens, int hidden, int vocab, void* stream);
+int tqk_remember_tokens(const int32_t* tokens, const int32_t* cu, const int32_t* seq_new, const int32_t* seq_slot, int32_t* last,
+                        int n_seqs, void* stream);
+int tqk_norm_add(float* h, const void* y, int act_dtype, const void* weight, int weight_dtype, float eps, void* copy, int n_tokens,
+                 int hidden, void* stream);
+int tqk_unary_act(const void* x, void* out, int act_dtype, long long n, int kind, float limit, float alpha, void* stream);
+int tqk_row_gate(const void* x, int act_dtype, const void* w, int w_dtype, float* out, int n_tokens, int hidden, void* stream);
+
+/* Attention with keys of key_dim and values of value_dim per head (attention_masked.hip).  tqk_normed_rope_store: a row of qkv is
+ * [heads * key_dim | kv_heads * key_dim | kv_heads * value_dim]; every query and key head is divided by its root mean square
+ * (eps inside the root) and multiplied by q_norm_w / k_norm_w [key_dim] (null: no norm), then its first rot_dim elements are
+ * rotated in halves by the angle table row tok_pos[t]; values become (1 - mix[0]) v + mix[0] mix_with[t] where mix_with
+ * [tokens, kv_heads * value_dim] is given, and are written to mix_keep (if given) as they go to the cache.  Pages: keys
+ * [n_pages, kv_heads, 64, key_dim], values [n_pages, kv_heads, value_dim, 64] with the places of tqk_rope_store.
+ * tqk_attention_masked: a query at position i sees j <= i with i - j < window or j < keep_first (window 0: all); scores
+ * scale q.k, then cap tanh(s / cap) if cap > 0; sink [heads] (or null) adds exp(sink_h) to the softmax's denominator.
+ * One wave per (token, head), float32 throughout; out [tokens, heads * value_dim]. */
+int tqk_normed_rope_store(const void* qkv, int act_dtype, const void* q_norm_w, const void* k_norm_w, int w_dtype, float eps,
+                          const float* cos_table, const float* sin_table, int rot_dim, int max_positions, const void* mix,
+                          const void* mix_with, void* mix_keep, const int32_t* tok_seq, const int32_t* tok_pos,
+                          const int32_t* page_table, int table_width, void* keys, void* values, void* q_out, int n_tokens,
+                          int n_heads, int n_kv_heads, int key_dim, int value_dim, int write_kv, void* stream);
+int tqk_attention_masked_max_dim(void);
+int tqk_attention_masked(const void* q, const void* keys, const void* values, int act_dtype, const int32_t* tok_seq,
+                         const int32_t* tok_pos, const int32_t* page_table, int table_width, int n_seqs, int n_pages, int window,
+                         int keep_first, float scale, float cap, const void* sink, int sink_dtype, void* out, int n_tokens,
+                         int n_heads, int n_kv_heads, int key_dim, int value_dim, void* stream);
 
 /* out[r] = lowest index of the largest value of logits[r, :]; scratch: at least
  * tqk_argmax_scratch_floats(n_rows, vocab) floats of device memory. */

@@ -203,7 +203,9 @@ void check_weights(const std::map<std::string, StoredTensor>& stored, const Tens
         auto it = stored.find(w.first);
         if (it == stored.end()) continue;
         const StoredTensor& st = it->second;
-        if (st.shape != w.second.shape) {
+        // a scalar (no dimensions) and a tensor of one element are the same thing: that is how a scalar is held
+        auto held_as = [](const std::vector<int64_t>& s) { return s.empty() ? std::vector<int64_t>{1} : s; };
+        if (held_as(st.shape) != held_as(w.second.shape)) {
             shape_lines.push_back("  Wrong shape: " + w.first + " is " + shape_text(st.shape) + ", expected " + shape_text(w.second.shape));
             Json e = Json::array();
             e.push(w.first);

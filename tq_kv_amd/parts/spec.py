@@ -77,6 +77,7 @@ class KVNeed:
     value_dim: Optional[int] = None
     key_page: Optional[Tuple[int, ...]] = None
     value_page: Optional[Tuple[int, ...]] = None
+    keep_first: int = 0         # with a window: the sequence's first positions that stay visible (their pages are kept)
 
     def pages(self):
         page = native.page_size()
@@ -86,7 +87,10 @@ class KVNeed:
 
     def to_json(self):
         key, value = self.pages()
-        return {"kind": "pages", "key_page": list(key), "value_page": list(value), "window": self.window}
+        j = {"kind": "pages", "key_page": list(key), "value_page": list(value), "window": self.window}
+        if self.keep_first:
+            j["keep_first"] = int(self.keep_first)
+        return j
 
 
 @dataclass(frozen=True)
@@ -110,8 +114,8 @@ def need_from_json(j):
     key, value = tuple(j["key_page"]), tuple(j["value_page"])
     page = native.page_size()
     if len(key) == 3 and len(value) == 3 and key[1] == page and value[2] == page and key[0] == value[0]:
-        return KVNeed(key[0], key[2], j.get("window"), None if value[1] == key[2] else value[1])
-    return KVNeed(window=j.get("window"), key_page=key, value_page=value)
+        return KVNeed(key[0], key[2], j.get("window"), None if value[1] == key[2] else value[1], keep_first=j.get("keep_first", 0))
+    return KVNeed(window=j.get("window"), key_page=key, value_page=value, keep_first=j.get("keep_first", 0))
 
 
 def need_to_json(need):

@@ -457,9 +457,44 @@ private:
                              q.data, (int)n, n_heads_, n_kv_heads_, head_dim_, value_dim_, write ? 1 : 0, c.stream);
     }
 
-    // attention of rows (sequence tok_seq[r], position tok_pos[r]) with the cap, the kept first positions and the sink
+    // Attention of rows (sequence tok_seq[r], position tok_pos[r]) with the cap, the kept first positions and the sink.  bfloat16 on the
+    // matrix cores where the sizes allow: steps of one token a sequence and a few chosen rows with a row's pages dealt out to
+    // partitions, other steps in tiles of consecutive queries; else the plain kernel, one wave per (row, head).
     void attend_masked(StepContext& c, const Tensor& q, const CacheEntry& entry, const StepContext::Table& table, const int32_t* tok_seq,
-                       const int32_t* tok_pos, Tensor& out) {
+                       const int32_t* tok_pos, Tensor& out, bool last_rows) {
+        const int n = (int)q.shape[0], n_pages = (int)entry.keys.shape[0];
+        const void* sink = sink_ ? sink_->t.data : nullptr;
+        const int sink_dtype = sink_ ? sink_->t.dtype : 0;
+        if (q.dtype == BF16 && K::attention_masked_mfma_supported.raw(head_dim_, value_dim_)) {
+            const bool rows = last_rows ? n <= DECODE_KERNEL_ROWS : c.all_decode;
+            if (rows && policy().decode_mfma) {
+                const int32_t* row_table = table.dev;
+                if (last_rows) {
+                    Tensor gathered = c.alloc(I32, {n, table.width});
+                    Tensor whole((void*)table.dev, I32, {c.n_seqs, table.width});
+                    k_gather_rows(c, whole, c.dev.last_seq, n, gathered);
+                    row_table = (const int32_t*)gathered.data;
+                }
+                const int n_parts = partitions(n, table.width);
+                Tensor part_out, part_ml;
+                if (n_parts > 1) {
+                    part_out = c.alloc(F32, {n, n_heads_, n_parts, value_dim_});
+                    part_ml = c.alloc(F32, {n, n_heads_, n_parts, 2});
+                }
+                K::attention_masked_mfma(q.data, entry.keys.data, entry.values.data, tok_pos, row_table, table.width, n_pages, window_, keep_first_, scale_,
+                                         cap_, sink, sink_dtype, nullptr, nullptr, nullptr, 0, n, n_parts, part_out.data, part_ml.data, out.data, n_heads_,
+                                         n_kv_heads_, head_dim_, value_dim_, c.stream);
+                return;
+            }
+            if (!rows && policy().prefill_mfma) {
+                const int tile = K::attention_masked_mfma_tile.raw();
+                const Tiles t = last_rows ? c.last_tiles(tile) : c.query_tiles(tile);
+                K::attention_masked_mfma(q.data, entry.keys.data, entry.values.data, tok_pos, table.dev, table.width, n_pages, window_, keep_first_, scale_,
+                                         cap_, sink, sink_dtype, t.seq, t.tok0, t.count, t.n, 0, 1, nullptr, nullptr, out.data, n_heads_, n_kv_heads_,
+                                         head_dim_, value_dim_, c.stream);
+                return;
+            }
+        }
         K::attention_masked(q.data, entry.keys.data, entry.values.data, q.dtype, tok_seq, tok_pos, table.dev, table.width, c.n_seqs,
                             (int)entry.keys.shape[0], window_, keep_first_, scale_, cap_, sink_ ? sink_->t.data : nullptr, sink_ ? sink_->t.dtype : 0,
                             out.data, (int)q.shape[0], n_heads_, n_kv_heads_, head_dim_, value_dim_, c.stream);
@@ -515,6 +550,15 @@ private:
                           c.stream);
     }
 
+    // how many partitions a row's pages are dealt out to in the kernels for steps of one token a sequence
+    int partitions(int n, int width) const {
+        const int q_blocks = (n_heads_ / n_kv_heads_ + 15) / 16;
+        const int groups = std::max(1, n * n_kv_heads_ * q_blocks);
+        int n_parts = std::max(1, std::min((width + 3) / 4, 256 / groups));
+        if (width > 1 && (long long)groups * width <= 640) n_parts = width;
+        return n_parts;
+    }
+
     void decode_kernel(StepContext& c, const Tensor& q, const CacheEntry& entry, const int32_t* tok_pos, const int32_t* table, int width,
                        Tensor& out) {
         const int n = (int)q.shape[0];
@@ -548,7 +592,7 @@ private:
     // tiled prompt kernel.
     void attend(StepContext& c, const Tensor& q, const CacheEntry& entry, const StepContext::Table& table, Tensor& out) {
         const int n = (int)q.shape[0], n_pages = (int)entry.keys.shape[0];
-        if (extras_) return attend_masked(c, q, entry, table, c.dev.tok_seq, c.dev.tok_pos, out);
+        if (extras_) return attend_masked(c, q, entry, table, c.dev.tok_seq, c.dev.tok_pos, out, false);
         if (q.dtype == BF16 && c.all_decode && policy().decode_mfma && K::attention_decode_supported.raw(head_dim_))
             return decode_kernel(c, q, entry, c.dev.tok_pos, table.dev, table.width, out);
         // (not for steps of one token per sequence: tiles of one query are what the plain kernel does anyway,
@@ -569,7 +613,7 @@ private:
     // keys and values of all the step's tokens.
     void attend_rows(StepContext& c, const Tensor& q, const CacheEntry& entry, const StepContext::Table& table, Tensor& out) {
         const int n = (int)q.shape[0], n_pages = (int)entry.keys.shape[0];
-        if (extras_) return attend_masked(c, q, entry, table, c.dev.last_seq, c.dev.last_pos, out);
+        if (extras_) return attend_masked(c, q, entry, table, c.dev.last_seq, c.dev.last_pos, out, true);
         if (q.dtype == BF16 && policy().decode_mfma && K::attention_decode_supported.raw(head_dim_) && c.n_last <= DECODE_KERNEL_ROWS) {
             // few rows: the decoding kernel shares a row's keys out over many blocks, where the prompt
             // kernel would walk them in one; a row is a sequence of its own to it

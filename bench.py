@@ -18,7 +18,9 @@ reference's prompt-inclusive figure goes into `end_to_end_tok_per_s`.
 `python bench.py --latent` is another measurement with a line of its own (the default workload above is untouched): the
 Nikasun design (attention through cached latents with a window, routed experts) at a few sizes that resemble a real
 model's layers, beside a Qwen2 shape of the same width, depth, heads and active feed-forward size: prompt pass and
-decoding of both, tokens a second.
+decoding of both, tokens a second.  `python bench.py --masked` does the same for the Sizudra design (attention with normed
+heads, mixed values, and in every other layer a score cap, a window that keeps the first positions and a sink; a pair
+embedding; norms on the parts' outputs; routed experts without a gate product).
 """
 import argparse
 import gc
@@ -45,7 +47,8 @@ def main():
     ap.add_argument("--no-tune", action="store_true", help="do not let the matrix library try its kernels for the prompt's size")
     ap.add_argument("--no-probe", action="store_true")
     ap.add_argument("--latent", action="store_true", help="measure the Nikasun design beside a Qwen2 shape of equal size instead of the default workload")
-    ap.add_argument("--latent-sizes", default="2048,4096", help="widths of the --latent comparison")
+    ap.add_argument("--latent-sizes", default="2048,4096", help="widths of the --latent and --masked comparisons")
+    ap.add_argument("--masked", action="store_true", help="measure the Sizudra design beside a Qwen2 shape of equal size instead of the default workload")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this library runs on one GPU; --gpus %d is not supported" % args.gpus)
@@ -150,7 +153,9 @@ def main():
 
     # -- another design beside the closest existing one -----------------------------------------------
     if args.latent:
-        return latent_comparison(args, torch, Model, Engine, note, timed_prefill, decode, random_prompts, release)
+        return design_comparison("nikasun", latent_shapes, args, torch, Model, Engine, note, timed_prefill, decode, random_prompts, release)
+    if args.masked:
+        return design_comparison("sizudra", masked_shapes, args, torch, Model, Engine, note, timed_prefill, decode, random_prompts, release)
 
     # -- the headline shape -------------------------------------------------------------------------
     raw = dict(catalog.find(args.shape))
@@ -310,12 +315,35 @@ def latent_shapes(width, layers=4):
                             "shared_ff": shared, "active_ff": active, "q_rank": mixer["q_rank"], "kv_rank": 512, "window": 1024}
 
 
-def latent_comparison(args, torch, Model, Engine, note, timed_prefill, decode, random_prompts, release):
+def masked_shapes(width, layers=4):
+    """A Sizudra configuration and a Qwen2 one of the same width, depth, heads, head size and active feed-forward products."""
+    heads, dim = width // 128, 128
+    kv_heads = max(1, heads // 4)
+    experts, top, ff = (32, 4, width // 2) if width <= 2048 else (64, 6, width // 4)
+    shared = 2 * ff
+    # an expert is two products, a gated feed-forward three: the dense size whose three products equal the active experts' two
+    active = 2 * (top * ff + shared) // 3 // 256 * 256
+    plain = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "rot": {"base": 10000.0, "dims": 64}, "v_mix": True}
+    second = dict(plain, softcap=30.0, mask={"size": 1024, "keep_first": 4})
+    moe = {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": ff}, "shared": {"ff": shared}}
+    lay = [{"type": "attention_2" if l % 2 else "attention", "mixer": second if l % 2 else plain,
+            "mlp": {"kind": "dense", "ff": active} if l == 0 else moe} for l in range(layers)]
+    sizudra = {"architecture": "Sizudra", "vocab": 32000, "width": width, "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 17}},
+               "norm": {"eps": 1e-5}, "layers": lay, "max_positions": 8192}
+    qwen2 = {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "hidden_act": "silu", "vocab_size": 32000, "hidden_size": width,
+             "intermediate_size": active, "num_hidden_layers": layers, "num_attention_heads": heads, "num_key_value_heads": kv_heads,
+             "head_dim": dim, "rms_norm_eps": 1e-5, "rope_theta": 10000.0, "max_position_embeddings": 8192, "tie_word_embeddings": False,
+             "use_sliding_window": True, "sliding_window": 1024, "max_window_layers": layers // 2}
+    return sizudra, qwen2, {"width": width, "layers": layers, "heads": heads, "kv_heads": kv_heads, "experts": experts, "top": top, "expert_ff": ff,
+                            "shared_ff": shared, "dense_ff": active, "window": 1024, "keep_first": 4}
+
+
+def design_comparison(design, shapes, args, torch, Model, Engine, note, timed_prefill, decode, random_prompts, release):
     prompt_len, out = 2048, {}
     for width in [int(x) for x in args.latent_sizes.split(",")]:
-        nikasun, qwen2, sizes = latent_shapes(width)
+        other, qwen2, sizes = shapes(width)
         row = {"sizes": sizes}
-        for name, raw in (("nikasun", nikasun), ("qwen2", qwen2)):
+        for name, raw in ((design, other), ("qwen2", qwen2)):
             note("width %d, %s: random weights" % (width, name))
             model = Model.random(raw, seed=0, dtype="bfloat16", device="cuda:0")
             engine = Engine(model, max_tokens=64 * (prompt_len + 256))
@@ -332,13 +360,13 @@ def latent_comparison(args, torch, Model, Engine, note, timed_prefill, decode, r
             engine = model = None
             release()
         for key in ("prefill_tok_s", "decode_b8_tok_s", "decode_b64_tok_s"):
-            row["ratio_" + key] = round(row["nikasun_" + key] / row["qwen2_" + key], 3)
+            row["ratio_" + key] = round(row[design + "_" + key] / row["qwen2_" + key], 3)
         out["width_%d" % width] = row
     first = out["width_%d" % int(args.latent_sizes.split(",")[0])]
-    print(json.dumps({"metric": "decode tok/s @ batch 8, Nikasun design at width %s" % args.latent_sizes.split(",")[0],
-                      "value": first["nikasun_decode_b8_tok_s"], "unit": "tokens/s", "n_gpus": 1, "steps": min(args.steps, 32), "warmup": 4,
-                      "ms_per_step": first["nikasun_decode_b8_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-                      "dtype": "bf16", "data": "synthetic", "config": {"model": "nikasun beside qwen2 at equal size", "prompt_len": prompt_len,
+    print(json.dumps({"metric": "decode tok/s @ batch 8, %s design at width %s" % (design.capitalize(), args.latent_sizes.split(",")[0]),
+                      "value": first[design + "_decode_b8_tok_s"], "unit": "tokens/s", "n_gpus": 1, "steps": min(args.steps, 32), "warmup": 4,
+                      "ms_per_step": first[design + "_decode_b8_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+                      "dtype": "bf16", "data": "synthetic", "config": {"model": design + " beside qwen2 at equal size", "prompt_len": prompt_len,
                                                                      "weights": "random"}, "comparison": out}))
     return 0
 

@@ -14,19 +14,16 @@
 //          position, window and first visible key.
 // Pages between the kept first positions and the window are passed over.  Sizes need not be those of a build:
 // key_dim <= 32 KB (a multiple of 8), value_dim <= 16 DB; what lies beyond a head's sizes is not loaded.
+#include <type_traits>
+
 #include "common.h"
 #include "tq_kernels.h"
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4_t;
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 namespace {
-
-union pack8 {
-    bf16x8_t v;
-    uint16_t u[8];
-    uint4 q;
-};
 
 struct MaskedArgs {
     const bf16_t *q, *keys, *values;
@@ -45,6 +42,32 @@ struct MaskedArgs {
 
 __device__ __forceinline__ float sink_of(const MaskedArgs& a, int head) {
     return (a.sink_f32 ? ((const float*)a.sink)[head] : to_float(((const bf16_t*)a.sink)[head])) * LOG2E;
+}
+
+// A 16-byte operand that lies beyond a head's size is zero.  The load itself is never under a condition (a branch around every load
+// would let none of them be under way together): it reads a place that is there, and the value is dropped.
+__device__ __forceinline__ bf16x8_t load_or_zero(const void* base, int offset_bytes, bool wanted) {
+    const bf16x8_t v = *reinterpret_cast<const bf16x8_t*>((const unsigned char*)base + (wanted ? offset_bytes : 0));
+    const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    return wanted ? v : zero;
+}
+
+// Eight probabilities of a lane as the second product's operand: bfloat16, two a word, built in registers (element i of the operand is
+// word i / 2, low half first).  The sum takes the rounded values.
+__device__ __forceinline__ uint32_t two_probabilities(float s0, float s1, float base, float& sum) {
+    const uint32_t b0 = float_to_bf16_bits(__builtin_amdgcn_exp2f(s0 - base)), b1 = float_to_bf16_bits(__builtin_amdgcn_exp2f(s1 - base));
+    sum += __uint_as_float(b0 << 16) + __uint_as_float(b1 << 16);
+    return b0 | (b1 << 16);
+}
+// the operand of values of a page's keys key0 + (2 pr + i / 4) 16 + 4 g + i % 4, those beyond `last` set to zero
+__device__ __forceinline__ bf16x8_t values_up_to(bf16x8_t v, int key0, int pr, int g, int last) {
+    u32x4_t w = __builtin_bit_cast(u32x4_t, v);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int j = key0 + (2 * pr + k / 2) * 16 + g * 4 + (k % 2) * 2;
+        w[k] &= (j > last ? 0u : 0xffffu) | (j + 1 > last ? 0u : 0xffff0000u);
+    }
+    return __builtin_bit_cast(bf16x8_t, w);
 }
 
 // tanh by one exponential: 1 - 2 / (e^(2x) + 1); exact at both ends (e^(2x) = inf gives 1, 0 gives -1)
@@ -114,12 +137,10 @@ void attention_masked_mfma_kernel(const MaskedArgs a) {
     for (int i = 0; i < DB; ++i) o[i] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 
     if (visit0 < n_visits) {
-        pack8 zero;
-        zero.q = make_uint4(0, 0, 0, 0);
         bf16x8_t bq[KB];
-        const bf16_t* qr = a.q + qrow * dk + g * 8;
+        const bf16_t* qr = a.q + qrow * dk;
 #pragma unroll
-        for (int kb = 0; kb < KB; ++kb) bq[kb] = (live && kb * 32 + g * 8 < dk) ? *reinterpret_cast<const bf16x8_t*>(qr + kb * 32) : zero.v;
+        for (int kb = 0; kb < KB; ++kb) bq[kb] = load_or_zero(qr, (kb * 32 + g * 8) * 2, live && kb * 32 + g * 8 < dk);
 
         const int32_t* pages = a.page_table + (size_t)seq * a.table_width;
         const size_t k_stride = (size_t)a.n_kv_heads * TQK_PAGE * dk, v_stride = (size_t)a.n_kv_heads * TQK_PAGE * dv;
@@ -138,12 +159,12 @@ void attention_masked_mfma_kernel(const MaskedArgs a) {
             for (int t = 0; t < 4; ++t)
 #pragma unroll
                 for (int kb = 0; kb < KB; ++kb)
-                    ka[t][kb] = kb * 32 + g * 8 < dk ? *reinterpret_cast<const bf16x8_t*>(kp + (size_t)(t * 16 + col) * dk + kb * 32 + g * 8) : zero.v;
+                    ka[t][kb] = load_or_zero(kp + (size_t)(t * 16 + col) * dk, (kb * 32 + g * 8) * 2, kb * 32 + g * 8 < dk);
 #pragma unroll
             for (int db = 0; db < DB; ++db)
 #pragma unroll
                 for (int pr = 0; pr < 2; ++pr)
-                    va[db][pr] = db * 16 + col < dv ? *reinterpret_cast<const bf16x8_t*>(vp + (size_t)(db * 16 + col) * TQK_PAGE + pr * 32 + g * 8) : zero.v;
+                    va[db][pr] = load_or_zero(vp, ((db * 16 + col) * TQK_PAGE + pr * 32 + g * 8) * 2, db * 16 + col < dv);
 
             floatx4_t s[4];
 #pragma unroll
@@ -171,33 +192,22 @@ void attention_masked_mfma_kernel(const MaskedArgs a) {
             const float alpha = __builtin_amdgcn_exp2f(m - base);
             m = mx;
             float psum = 0.f;
-            pack8 pb[2];
+            u32x4_t pw[2];
 #pragma unroll
             for (int t = 0; t < 4; ++t)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const float p = __builtin_amdgcn_exp2f(s[t][r] - base);
-                    const uint16_t pbits = float_to_bf16_bits(p);
-                    psum += __uint_as_float(((uint32_t)pbits) << 16);
-                    pb[t / 2].u[(t % 2) * 4 + r] = pbits;
-                }
+                for (int h = 0; h < 2; ++h) pw[t / 2][(t % 2) * 2 + h] = two_probabilities(s[t][2 * h], s[t][2 * h + 1], base, psum);
+            const bf16x8_t pb[2] = {__builtin_bit_cast(bf16x8_t, pw[0]), __builtin_bit_cast(bf16x8_t, pw[1])};
             l = l * alpha + psum;
+            // beyond the last position of the step nothing has been written yet: whatever lies there must not meet a zero
+            const bool beyond = key0 + TQK_PAGE - 1 > pos_max;
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
                 o[db][0] *= alpha; o[db][1] *= alpha; o[db][2] *= alpha; o[db][3] *= alpha;
 #pragma unroll
                 for (int pr = 0; pr < 2; ++pr) {
-                    pack8 av;
-                    av.v = va[db][pr];
-                    if (key0 + TQK_PAGE - 1 > pos_max) {
-                        // beyond the last position of the step nothing has been written yet: whatever lies there must not meet a zero
-#pragma unroll
-                        for (int i = 0; i < 8; ++i) {
-                            const int j = key0 + (2 * pr + i / 4) * 16 + g * 4 + (i % 4);
-                            if (j > pos_max) av.u[i] = 0;
-                        }
-                    }
-                    o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av.v, pb[pr].v, o[db], 0, 0, 0);
+                    const bf16x8_t av = beyond ? values_up_to(va[db][pr], key0, pr, g, pos_max) : va[db][pr];
+                    o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, pb[pr], o[db], 0, 0, 0);
                 }
             }
         }
@@ -280,6 +290,203 @@ void attention_masked_mfma_kernel(const MaskedArgs a) {
     }
 }
 
+// Tiles, with a page staged once for a block.  A block of four waves takes one kv head and a tile of consecutive queries
+// of one sequence: its waves are min(4, heads of the group) query heads times 4 / that many sub-tiles of 16 CT queries
+// (CT = 2; a group of one head: 128 queries a block; of two: 64; of four or more: 32, the further heads in further
+// blocks).  A wave holds CT sets of 16 columns, so that what it reads of a page from LDS serves CT products.  Every
+// thread brings its pieces of the next page's keys and values into registers while the block computes on the page that
+// lies in LDS (two pages under way were measured no faster; rows padded by 16 bytes, so that the 16 rows a load of the matrix cores' operands touches fall on
+// different banks); a wave passes over a page none of its queries sees.  Sizes up to 128 and 128.
+template <int KB, int DB, int CT>
+__global__ __launch_bounds__(4 * TQK_WAVE) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void attention_masked_block_kernel(const MaskedArgs a) {
+    constexpr int KS_MAX = KB * 64 + 16, VS = 2 * TQK_PAGE + 16;        // bytes of a key row and of a value row in LDS
+    constexpr int VJ = (DB + 1) / 2;                                        // pieces of values a thread brings
+    constexpr int SUB = 16 * CT;                                            // queries of a wave
+    __shared__ __attribute__((aligned(16))) unsigned char lds_k[TQK_PAGE * KS_MAX];
+    __shared__ __attribute__((aligned(16))) unsigned char lds_v[DB * 16 * VS];
+    const int tid = threadIdx.x, wave = tid / TQK_WAVE, lane = tid % TQK_WAVE;
+    const int col = lane % 16, g = lane / 16;
+    const int n_rep = a.n_heads / a.n_kv_heads;
+    const int dk = a.dk, dv = a.dv, ks = dk * 2 + 16;
+    const int hpb = min(n_rep, 4), sph = 4 / hpb, chunks = (n_rep + hpb - 1) / hpb;
+    const int kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
+    const int tile = blockIdx.x;
+    const int seq = a.tile_seq[tile], tok0 = a.tile_tok0[tile], count = a.tile_count[tile];
+    const int pos0 = __builtin_amdgcn_readfirstlane(a.tok_pos[tok0]);
+
+    // the wave's head and sub-tile; a wave without either still brings pages in
+    const int rep = chunk * hpb + wave % hpb, sub = wave / hpb;
+    const bool active = rep < n_rep && sub < sph && sub * SUB < count;
+    const int head = kvh * n_rep + (rep < n_rep ? rep : 0);
+    const int w_first = pos0 + sub * SUB, w_max = min(pos0 + count - 1, w_first + SUB - 1);
+    bool live[CT];
+    int pos_c[CT], lo_c[CT];
+    size_t qrow[CT];
+    const int window = a.window;
+    const int kept = window > 0 ? a.keep_first : 0;
+#pragma unroll
+    for (int c = 0; c < CT; ++c) {
+        const int i = sub * SUB + c * 16 + col;
+        live[c] = active && i < count;
+        pos_c[c] = live[c] ? pos0 + i : w_first;
+        lo_c[c] = window > 0 ? max(0, pos_c[c] - window + 1) : 0;
+        qrow[c] = (size_t)(tok0 + (live[c] ? i : 0)) * a.n_heads + head;
+    }
+    const int w_lo_min = window > 0 ? max(0, w_first - window + 1) : 0, w_lo_max = window > 0 ? max(0, w_max - window + 1) : 0;
+    const int lo_min = window > 0 ? max(0, pos0 - window + 1) : 0;
+    const int pos_max = pos0 + count - 1;
+    const float scale = a.scale, cap = a.cap;
+    const float scale2 = scale * LOG2E;
+    const float cap2 = cap * LOG2E, scale_over_cap = cap > 0.f ? scale / cap : 0.f;
+
+    const int first_win_page = lo_min / TQK_PAGE, last_page = pos_max / TQK_PAGE;
+    const int kept_pages = min((kept + TQK_PAGE - 1) / TQK_PAGE, first_win_page);
+    const int n_visits = kept_pages + last_page - first_win_page + 1;
+
+    // where the thread's pieces of a page (16 bytes each) come from and go to
+    int k_src[KB], k_dst[KB], v_src[VJ], v_dst[VJ];
+    const int k_per_row = dk / 8;
+#pragma unroll
+    for (int j = 0; j < KB; ++j) {
+        const int p = tid + 256 * j;
+        const int pk = p < 8 * dk ? p : tid % (8 * dk);       // a piece beyond the page: one that is there, once more (the same bytes to the same place)
+        k_src[j] = pk;
+        k_dst[j] = (pk / k_per_row) * ks + (pk % k_per_row) * 16;
+    }
+#pragma unroll
+    for (int j = 0; j < VJ; ++j) {
+        const int p = tid + 256 * j;
+        const int pv = p < 8 * dv ? p : tid % (8 * dv);
+        v_src[j] = pv;
+        v_dst[j] = (pv / 8) * VS + (pv % 8) * 16;
+    }
+
+    float m[CT], l[CT];
+    floatx4_t o[CT][DB];
+    bf16x8_t bq[CT][KB];
+#pragma unroll
+    for (int c = 0; c < CT; ++c) {
+        m[c] = -INFINITY;
+        l[c] = 0.f;
+        if (a.sink && active) { m[c] = sink_of(a, head); l[c] = (g == 0) ? 1.f : 0.f; }       // l is summed over a column's four lanes at the end
+#pragma unroll
+        for (int i = 0; i < DB; ++i) o[c][i] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+        const bf16_t* qr = a.q + qrow[c] * dk;
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) bq[c][kb] = load_or_zero(qr, (kb * 32 + g * 8) * 2, live[c] && kb * 32 + g * 8 < dk);
+    }
+
+    const int32_t* pages = a.page_table + (size_t)seq * a.table_width;
+    const size_t k_stride = (size_t)a.n_kv_heads * TQK_PAGE * dk, v_stride = (size_t)a.n_kv_heads * TQK_PAGE * dv;
+    auto page_of = [&](int visit) { return visit < kept_pages ? visit : first_win_page + (visit - kept_pages); };
+    uint4 k_reg[KB], v_reg[VJ];
+    auto fetch = [&](int visit) {
+        const int page = __builtin_amdgcn_readfirstlane(pages[page_of(visit)]);
+        if (page < 0) return;                           // nothing of it is visible to anyone: what LDS then holds is not looked at
+        const uint4* kp = reinterpret_cast<const uint4*>(a.keys + (size_t)page * k_stride + (size_t)kvh * TQK_PAGE * dk);
+        const uint4* vp = reinterpret_cast<const uint4*>(a.values + (size_t)page * v_stride + (size_t)kvh * TQK_PAGE * dv);
+#pragma unroll
+        for (int j = 0; j < KB; ++j) k_reg[j] = kp[k_src[j]];
+#pragma unroll
+        for (int j = 0; j < VJ; ++j) v_reg[j] = vp[v_src[j]];
+    };
+    fetch(0);
+    for (int visit = 0; visit < n_visits; ++visit) {
+        const int pg = page_of(visit);
+        const int page = __builtin_amdgcn_readfirstlane(pages[pg]);
+        __syncthreads();                                // everyone has done with the page before
+#pragma unroll
+        for (int j = 0; j < KB; ++j) *reinterpret_cast<uint4*>(lds_k + k_dst[j]) = k_reg[j];
+#pragma unroll
+        for (int j = 0; j < VJ; ++j) *reinterpret_cast<uint4*>(lds_v + v_dst[j]) = v_reg[j];
+        __syncthreads();
+        if (visit + 1 < n_visits) fetch(visit + 1);
+        const int key0 = pg * TQK_PAGE;
+        // does any of the wave's queries see any of the page's keys
+        if (!active || page < 0 || key0 > w_max || !(key0 + TQK_PAGE > w_lo_min || key0 < kept)) continue;
+        const bool inside = key0 + TQK_PAGE - 1 <= w_first && (key0 >= w_lo_max || key0 + TQK_PAGE <= kept);
+
+        // scores^T for the page's four groups of 16 keys, a group's keys read once for all of the wave's columns
+        floatx4_t s[CT][4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            bf16x8_t ka[KB];
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+                ka[kb] = load_or_zero(lds_k, (t * 16 + col) * ks + (kb * 32 + g * 8) * 2, kb * 32 + g * 8 < dk);
+#pragma unroll
+            for (int c = 0; c < CT; ++c) {
+                s[c][t] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb) s[c][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[kb], bq[c][kb], s[c][t], 0, 0, 0);
+            }
+        }
+        bf16x8_t pb[CT][2];
+        float alpha[CT];
+#pragma unroll
+        for (int c = 0; c < CT; ++c) {
+            float mx = m[c];
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int j = key0 + t * 16 + g * 4 + r;
+                    float v = cap > 0.f ? cap2 * tanh_fast(s[c][t][r] * scale_over_cap) : s[c][t][r] * scale2;
+                    if (!inside && !(j <= pos_c[c] && (j >= lo_c[c] || j < kept))) v = -INFINITY;
+                    s[c][t][r] = v;
+                    mx = fmaxf(mx, v);
+                }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, TQK_WAVE));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, TQK_WAVE));
+            const float base = mx == -INFINITY ? 0.f : mx;      // a column that has met no key it sees yet
+            alpha[c] = __builtin_amdgcn_exp2f(m[c] - base);
+            m[c] = mx;
+            float psum = 0.f;
+            u32x4_t pw[2];
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int h = 0; h < 2; ++h) pw[t / 2][(t % 2) * 2 + h] = two_probabilities(s[c][t][2 * h], s[c][t][2 * h + 1], base, psum);
+            pb[c][0] = __builtin_bit_cast(bf16x8_t, pw[0]);
+            pb[c][1] = __builtin_bit_cast(bf16x8_t, pw[1]);
+            l[c] = l[c] * alpha[c] + psum;
+        }
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+            bf16x8_t av[2];
+#pragma unroll
+            for (int pr = 0; pr < 2; ++pr) {
+                av[pr] = load_or_zero(lds_v, (db * 16 + col) * VS + (pr * 32 + g * 8) * 2, db * 16 + col < dv);
+                // beyond the last position of the step nothing has been written yet: whatever lies there must not meet a zero
+                if (key0 + TQK_PAGE - 1 > pos_max) av[pr] = values_up_to(av[pr], key0, pr, g, pos_max);
+            }
+#pragma unroll
+            for (int c = 0; c < CT; ++c) {
+                o[c][db][0] *= alpha[c]; o[c][db][1] *= alpha[c]; o[c][db][2] *= alpha[c]; o[c][db][3] *= alpha[c];
+#pragma unroll
+                for (int pr = 0; pr < 2; ++pr) o[c][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[pr], pb[c][pr], o[c][db], 0, 0, 0);
+            }
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < CT; ++c) {
+        float lc = l[c];
+        lc += __shfl_xor(lc, 16, TQK_WAVE);
+        lc += __shfl_xor(lc, 32, TQK_WAVE);
+        if (!live[c]) continue;
+        bf16_t* po = a.out + qrow[c] * dv;
+        const float inv = 1.f / lc;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int e = db * 16 + g * 4 + r;
+                if (e < dv) po[e] = from_float<bf16_t>(o[c][db][r] * inv);
+            }
+    }
+}
+
 // out[row, :] = sum_p 2^(m_p - M) o_p / (sum_p 2^(m_p - M) l_p + 2^(sink - M)), partitions in order
 __global__ void attention_masked_merge_kernel(const float* __restrict__ part_out, const float* __restrict__ part_ml, int n_parts, int dv, int n_heads,
                                               const void* __restrict__ sink, int sink_f32, bf16_t* __restrict__ out) {
@@ -312,8 +519,14 @@ __global__ void attention_masked_merge_kernel(const float* __restrict__ part_out
 template <int KB, int DB>
 int launch_masked(const MaskedArgs& a, bool tiles, int n_tiles, int n_rows, hipStream_t s) {
     if (tiles) {
-        dim3 grid(n_tiles, (a.n_heads + 3) / 4);
-        attention_masked_mfma_kernel<KB, DB, 4, true><<<grid, 4 * TQK_WAVE, 0, s>>>(a);
+        if constexpr (KB <= 4 && DB <= 8) {
+            const int n_rep = a.n_heads / a.n_kv_heads, hpb = n_rep < 4 ? n_rep : 4;
+            dim3 grid(n_tiles, a.n_kv_heads * ((n_rep + hpb - 1) / hpb));
+            attention_masked_block_kernel<KB, DB, 2><<<grid, 4 * TQK_WAVE, 0, s>>>(a);
+        } else {
+            dim3 grid(n_tiles, (a.n_heads + 3) / 4);
+            attention_masked_mfma_kernel<KB, DB, 4, true><<<grid, 4 * TQK_WAVE, 0, s>>>(a);
+        }
     } else {
         dim3 grid(a.n_parts, a.n_kv_heads * a.q_blocks, n_rows);
         // a partition per page of the table: a block has one page to read, and one wave does it
@@ -336,7 +549,12 @@ int launch_masked_dv(const MaskedArgs& a, bool tiles, int n_tiles, int n_rows, h
 extern "C" int tqk_attention_masked_mfma_supported(int key_dim, int value_dim) {
     return key_dim > 0 && key_dim % 8 == 0 && key_dim <= 256 && value_dim > 0 && value_dim <= 256;
 }
-extern "C" int tqk_attention_masked_mfma_tile(void) { return 16; }
+/* queries per tile for steps of several tokens a sequence: 32 for each sub-tile a block's waves make of a tile */
+extern "C" int tqk_attention_masked_mfma_tile(int n_heads, int n_kv_heads, int key_dim, int value_dim) {
+    if (key_dim > 128 || value_dim > 128 || n_kv_heads <= 0) return 16;
+    const int n_rep = n_heads / n_kv_heads;
+    return 32 * (4 / (n_rep < 4 ? (n_rep > 0 ? n_rep : 1) : 4));
+}
 
 /* n_tiles > 0: tiles of up to 16 consecutive queries of one sequence (tile_seq, tile_tok0, tile_count on the device; tok_pos and q by
  * packed token, page_table by sequence of the step).  Else rows: row r is a token of its own at position tok_pos[r] whose pages are
@@ -367,7 +585,7 @@ extern "C" int tqk_attention_masked_mfma(const void* q, const void* keys, const 
     a.sink = sink; a.sink_f32 = sink_dtype == TQK_F32;
     a.n_parts = tiles ? 1 : n_parts; a.n_heads = n_heads; a.n_kv_heads = n_kv_heads;
     a.q_blocks = (n_heads / n_kv_heads + 15) / 16;
-    TQK_REQUIRE((long long)n_kv_heads * a.q_blocks <= 65535 && (n_heads + 3) / 4 <= 65535, "tqk_attention_masked_mfma: grid too large");
+    TQK_REQUIRE((long long)n_kv_heads * a.q_blocks <= 65535 && n_heads <= 65535, "tqk_attention_masked_mfma: grid too large");
     a.dk = key_dim; a.dv = value_dim;
     a.tile_seq = tile_seq; a.tile_tok0 = tile_tok0; a.tile_count = tile_count;
     a.part_out = (float*)part_out; a.part_ml = (float*)part_ml; a.out = (bf16_t*)out;

@@ -36,7 +36,8 @@ def main(argv=None):
     from .engine import Engine, Model
 
     os.makedirs(args.out, exist_ok=True)
-    model = Model.from_dir(args.model, dtype=args.dtype, device="cuda")
+    # tensors the model does not use are named in a warning and otherwise left alone: a replay is about the steps
+    model = Model.from_dir(args.model, dtype=args.dtype, device="cuda", strict=False)
     # every live request may end in a page that is partly used, and a request may be as short as one token: room for
     # the tokens in whole pages plus a page for each of some hundred requests
     slots = 256

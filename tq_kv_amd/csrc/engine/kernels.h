@@ -67,7 +67,7 @@ TQ_QUERY(int, moe_tile_rows);
 TQ_QUERY(int, grouped_supported, int);
 TQ_KERNEL(moe_product_mfma, cptr, ci32, cptr, long long, void*, int, int, int, int, float, float, ci32, ci32, ci32, ci32, int, int, void*);
 TQ_KERNEL(head_product, cptr, int, long long, long long, cptr, void*, int, long long, long long, cf32, int, int, int, int, void*);
-TQ_KERNEL(moe_route, cptr, int, cptr, int, int, int, int, float, int, int32_t*, float*, int, void*);
+TQ_KERNEL(moe_route, cptr, int, cptr, int, int, int, int, float, int, int32_t*, float*, cptr, float*, int, void*);
 TQ_KERNEL(moe_group, ci32, int, int, int, int, int32_t*, int32_t*, int32_t*, int32_t*, int32_t*, int32_t*, void*);
 TQ_KERNEL(moe_product, cptr, int, ci32, cptr, int, long long, void*, int, int, int, int, float, float, ci32, ci32, ci32, ci32, int, void*);
 TQ_KERNEL(moe_combine, cptr, int, ci32, cf32, int, cptr, cf32, void*, int, int, void*);

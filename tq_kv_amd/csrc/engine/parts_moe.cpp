@@ -139,15 +139,17 @@ public:
         int32_t* tile_expert = (int32_t*)tiles.data;
         int32_t* tile_row0 = tile_expert + max_tiles;
         int32_t* tile_rows = tile_row0 + max_tiles;
+        // the shared expert's gate rides along with the router where both weights are of one type
+        Tensor shared_scale;
+        const bool gate_in_route = shared_gate_ && shared_gate_->t.dtype == router_->t.dtype;
+        if (shared_gate_) shared_scale = c.alloc(F32, {n});
         K::moe_route(x.x.data, dtype, router_->t.data, router_->t.dtype, n_experts_, (int)hidden_, top_, router_scale_, renormalize_ ? 1 : 0, (int32_t*)idx.data,
-                     (float*)weight.data, (int)n, c.stream);
+                     (float*)weight.data, gate_in_route ? shared_gate_->t.data : nullptr, gate_in_route ? (float*)shared_scale.data : nullptr, (int)n, c.stream);
         K::moe_group((const int32_t*)idx.data, (int)n, top_, n_experts_, tile_m, (int32_t*)pair_pos.data, (int32_t*)sorted_tok.data, tile_expert, tile_row0,
                      tile_rows, (int32_t*)n_tiles.data, c.stream);
         Tensor shared_out;
         if (shared_) shared_out = shared_->forward(c, x, nullptr);
-        Tensor shared_scale;
-        if (shared_gate_) {
-            shared_scale = c.alloc(F32, {n});
+        if (shared_gate_ && !gate_in_route) {
             K::row_gate(x.x.data, dtype, shared_gate_->t.data, shared_gate_->t.dtype, (float*)shared_scale.data, (int)n, (int)hidden_, c.stream);
         }
         // an expert's first product: gate and up side by side, or up alone with the gate's function of it

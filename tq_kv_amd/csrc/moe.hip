@@ -27,13 +27,14 @@
 template <typename TA, typename TW>
 __global__ __launch_bounds__(MOE_ROUTE_WAVES * TQK_WAVE)
 void moe_route_kernel(const TA* __restrict__ x, const TW* __restrict__ w, int n_experts, int hidden, int top, float scale, int renormalize,
-                      int32_t* __restrict__ idx, float* __restrict__ weight) {
+                      int32_t* __restrict__ idx, float* __restrict__ weight, const TW* __restrict__ gate_w, float* __restrict__ gate_out) {
     __shared__ float z[MOE_MAX_EXPERTS];
     const int wave = threadIdx.x / TQK_WAVE, lane = threadIdx.x % TQK_WAVE;
     const int t = blockIdx.x;
     const TA* xr = x + (size_t)t * hidden;
-    for (int e = wave; e < n_experts; e += MOE_ROUTE_WAVES) {
-        const TW* wr = w + (size_t)e * hidden;
+    // one row more where a gate is given: sigmoid(x . gate_w) per token, which rides along with the experts' dot products
+    for (int e = wave; e < n_experts + (gate_w ? 1 : 0); e += MOE_ROUTE_WAVES) {
+        const TW* wr = e < n_experts ? w + (size_t)e * hidden : gate_w;
         float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
         int i = lane;
         if (sizeof(TA) == 2 && sizeof(TW) == 2 && hidden % 8 == 0) {
@@ -61,7 +62,10 @@ void moe_route_kernel(const TA* __restrict__ x, const TW* __restrict__ w, int n_
         }
         for (; i < hidden; i += TQK_WAVE) d0 = fmaf(to_float(xr[i]), to_float(wr[i]), d0);
         const float dot = wave_sum((d0 + d1) + (d2 + d3));
-        if (lane == 0) z[e] = dot;
+        if (lane == 0) {
+            if (e < n_experts) z[e] = dot;
+            else gate_out[t] = 1.f / (1.f + expf(-dot));
+        }
     }
     __syncthreads();
     if (wave != 0) return;
@@ -242,14 +246,15 @@ extern "C" int tqk_moe_tile_rows(void) { return MOE_TM; }
 extern "C" int tqk_moe_max_tiles(int n_pairs, int n_experts, int tile_m) { return (n_pairs + tile_m - 1) / tile_m + n_experts; }
 
 extern "C" int tqk_moe_route(const void* x, int act_dtype, const void* w_router, int w_dtype, int n_experts, int hidden, int top, float scale,
-                             int renormalize, int32_t* idx, float* weight, int n_tokens, void* stream) {
+                             int renormalize, int32_t* idx, float* weight, const void* gate_w, float* gate_out, int n_tokens, void* stream) {
     TQK_REQUIRE(x && w_router && idx && weight, "tqk_moe_route: null pointer");
     TQK_REQUIRE(n_experts > 0 && n_experts <= MOE_MAX_EXPERTS, "tqk_moe_route: %d experts, the kernel takes 1 to %d", n_experts, MOE_MAX_EXPERTS);
     TQK_REQUIRE(top > 0 && top <= n_experts && hidden > 0 && n_tokens >= 0, "tqk_moe_route: bad sizes (top %d of %d experts)", top, n_experts);
+    TQK_REQUIRE(!gate_w || gate_out, "tqk_moe_route: a gate without a place for its values");
     if (n_tokens == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
 #define TQK_ROUTE(TA, TW) \
-    moe_route_kernel<TA, TW><<<n_tokens, MOE_ROUTE_WAVES * TQK_WAVE, 0, s>>>((const TA*)x, (const TW*)w_router, n_experts, hidden, top, scale, renormalize, idx, weight)
+    moe_route_kernel<TA, TW><<<n_tokens, MOE_ROUTE_WAVES * TQK_WAVE, 0, s>>>((const TA*)x, (const TW*)w_router, n_experts, hidden, top, scale, renormalize, idx, weight, (const TW*)gate_w, gate_out)
     if (act_dtype == TQK_F32 && w_dtype == TQK_F32) TQK_ROUTE(float, float);
     else if (act_dtype == TQK_F32 && w_dtype == TQK_BF16) TQK_ROUTE(float, bf16_t);
     else if (act_dtype == TQK_BF16 && w_dtype == TQK_F32) TQK_ROUTE(bf16_t, float);

@@ -62,6 +62,55 @@ void norm_add_kernel(float* __restrict__ h, const TA* __restrict__ y, const TW* 
     }
 }
 
+// The same for bfloat16 rows whose length is a multiple of 8 and at most 2048 NCH: a thread takes 8 neighbouring elements at a time with
+// 16-byte loads and keeps its part of y in registers between the sum of squares and the update, so a row is read once.
+template <typename TW, int NCH>
+__global__ __launch_bounds__(256)
+void norm_add_vec_kernel(float* __restrict__ h, const bf16_t* __restrict__ y, const TW* __restrict__ w, float eps, bf16_t* __restrict__ copy, int hidden) {
+    __shared__ float scratch[4];
+    const int t = blockIdx.x;
+    float yv[NCH][8];
+    float ss = 0.f;
+    if (y) {
+#pragma unroll
+        for (int k = 0; k < NCH; ++k) {
+            const int i = (threadIdx.x + k * 256) * 8;
+            if (i < hidden) {
+                const uint4 raw = *reinterpret_cast<const uint4*>(y + (size_t)t * hidden + i);
+                const uint32_t u[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) { yv[k][2 * j] = __uint_as_float(u[j] << 16); yv[k][2 * j + 1] = __uint_as_float(u[j] & 0xffff0000u); }
+#pragma unroll
+                for (int j = 0; j < 8; ++j) ss = fmaf(yv[k][j], yv[k][j], ss);
+            }
+        }
+    }
+    float inv = 1.f;
+    if (y && w) inv = 1.f / sqrtf(block_sum(ss, scratch) / (float)hidden + eps);
+#pragma unroll
+    for (int k = 0; k < NCH; ++k) {
+        const int i = (threadIdx.x + k * 256) * 8;
+        if (i >= hidden) continue;
+        float* hr = h + (size_t)t * hidden + i;
+        float4 a = *reinterpret_cast<const float4*>(hr), b = *reinterpret_cast<const float4*>(hr + 4);
+        float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+        if (y) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] += w ? yv[k][j] * inv * to_float(w[i + j]) : yv[k][j];
+            *reinterpret_cast<float4*>(hr) = make_float4(v[0], v[1], v[2], v[3]);
+            *reinterpret_cast<float4*>(hr + 4) = make_float4(v[4], v[5], v[6], v[7]);
+        }
+        if (copy) {
+            uint4 out;
+            out.x = float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
+            out.y = float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
+            out.z = float_to_bf16_bits(v[4]) | ((uint32_t)float_to_bf16_bits(v[5]) << 16);
+            out.w = float_to_bf16_bits(v[6]) | ((uint32_t)float_to_bf16_bits(v[7]) << 16);
+            *reinterpret_cast<uint4*>(copy + (size_t)t * hidden + i) = out;
+        }
+    }
+}
+
 template <typename TA>
 __global__ void unary_act_kernel(const TA* __restrict__ x, TA* __restrict__ out, long long n, int kind, float limit, float alpha) {
     const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -111,6 +160,14 @@ extern "C" int tqk_norm_add(float* h, const void* y, int act_dtype, const void* 
     TQK_REQUIRE(n_tokens >= 0 && hidden > 0, "tqk_norm_add: bad sizes");
     if (n_tokens == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
+    if (act_dtype == TQK_BF16 && hidden % 8 == 0 && hidden <= 8192 && ((((uintptr_t)h) | ((uintptr_t)y) | ((uintptr_t)copy)) & 15) == 0) {
+        // (the weight's type only matters where there is a weight)
+#define TQK_NAV(TW, NCH) norm_add_vec_kernel<TW, NCH><<<n_tokens, 256, 0, s>>>(h, (const bf16_t*)y, (const TW*)weight, eps, (bf16_t*)copy, hidden)
+        if (weight && weight_dtype == TQK_F32) { if (hidden <= 2048) TQK_NAV(float, 1); else if (hidden <= 4096) TQK_NAV(float, 2); else TQK_NAV(float, 4); }
+        else { if (hidden <= 2048) TQK_NAV(bf16_t, 1); else if (hidden <= 4096) TQK_NAV(bf16_t, 2); else TQK_NAV(bf16_t, 4); }
+#undef TQK_NAV
+        return tqk_check_launch("tqk_norm_add");
+    }
 #define TQK_NA(TA, TW) norm_add_kernel<TA, TW><<<n_tokens, 256, 0, s>>>(h, (const TA*)y, (const TW*)weight, eps, (TA*)copy, hidden)
     if (act_dtype == TQK_F32 && weight_dtype == TQK_F32) TQK_NA(float, float);
     else if (act_dtype == TQK_F32 && weight_dtype == TQK_BF16) TQK_NA(float, bf16_t);

@@ -234,13 +234,14 @@ int tqk_latent_values(const float* o, const void* w_uv, int w_dtype, const float
  * tile times its expert's weight (w + expert * expert_stride: [N, K], gated: gate rows then up rows [2 N, K]) into
  * y [pairs, N]; gated 0: the product alone, 1: gate and up, 2: one product [N, K] with the gate's function of it alone (u = 1:
  * relu2 gives max(z, 0)^2).  tqk_moe_route with renormalize: the chosen weights are divided by their sum (the softmax over
- * the chosen logits alone).  tqk_moe_combine: out[t] = sum_k weight[t, k] y[pair_pos[t, k]] + shared_scale[t] * shared[t]
+ * the chosen logits alone); with gate_w [hidden] (of the router's type, or null) it also writes gate_out[t] = sigmoid(x[t] . gate_w).
+ * tqk_moe_combine: out[t] = sum_k weight[t, k] y[pair_pos[t, k]] + shared_scale[t] * shared[t]
  * (shared may be null; shared_scale null: 1). */
 int tqk_moe_max_experts(void);
 int tqk_moe_tile_rows(void);
 int tqk_moe_max_tiles(int n_pairs, int n_experts, int tile_m);
 int tqk_moe_route(const void* x, int act_dtype, const void* w_router, int w_dtype, int n_experts, int hidden, int top, float scale,
-                  int renormalize, int32_t* idx, float* weight, int n_tokens, void* stream);
+                  int renormalize, int32_t* idx, float* weight, const void* gate_w, float* gate_out, int n_tokens, void* stream);
 int tqk_moe_group(const int32_t* idx, int n_tokens, int top, int n_experts, int tile_m, int32_t* pair_pos, int32_t* sorted_tok,
                   int32_t* tile_expert, int32_t* tile_row0, int32_t* tile_rows, int32_t* n_tiles, void* stream);
 int tqk_moe_product(const void* x, int act_dtype, const int32_t* x_rows, const void* w, int w_dtype, long long expert_stride, void* y,

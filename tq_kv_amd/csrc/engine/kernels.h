@@ -71,7 +71,7 @@ TQ_KERNEL(moe_route, cptr, int, cptr, int, int, int, int, float, int, int32_t*, 
 TQ_KERNEL(moe_group, ci32, int, int, int, int, int32_t*, int32_t*, int32_t*, int32_t*, int32_t*, int32_t*, void*);
 TQ_KERNEL(moe_product, cptr, int, ci32, cptr, int, long long, void*, int, int, int, int, float, float, ci32, ci32, ci32, ci32, int, void*);
 TQ_KERNEL(moe_combine, cptr, int, ci32, cf32, int, cptr, cf32, void*, int, int, void*);
-TQ_KERNEL(pair_embed, cptr, int, int, long long, long long, ci32, ci32, ci32, ci32, ci32, ci32, float*, int, int, int, void*);
+TQ_KERNEL(pair_embed, cptr, int, int, long long, long long, ci32, ci32, ci32, ci32, ci32, int32_t*, float*, int, int, int, void*, int, void*);
 TQ_KERNEL(remember_tokens, ci32, ci32, ci32, ci32, int32_t*, int, void*);
 TQ_KERNEL(norm_add, float*, cptr, int, cptr, int, float, void*, int, int, void*);
 TQ_KERNEL(unary_act, cptr, void*, int, long long, int, float, float, void*);

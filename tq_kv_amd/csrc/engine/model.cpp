@@ -153,9 +153,16 @@ Tensor Model::forward(StepContext& c, const CacheStore& cache, float* out) {
                  nullptr, c.stream);
     }
     if (stream_position_) {
-        if (stream_state_entry_ >= 0) stream_position_->add_to_stream_with(c, h, cache.entry(stream_state_entry_));
+        // a first block without a norm in front of it reads the stream itself: the part writes that copy too where it offers to
+        bool copied = false;
+        if (stream_state_entry_ >= 0 && !firsts[0] && c.act_dtype == BF16 && stream_position_->writes_stream_copy()) {
+            stream.copy = c.alloc(BF16, {c.n_tokens, s.hidden_size});
+            stream_position_->add_to_stream_copy(c, h, cache.entry(stream_state_entry_), stream.copy);
+            copied = true;
+        } else if (stream_state_entry_ >= 0) stream_position_->add_to_stream_with(c, h, cache.entry(stream_state_entry_));
         else stream_position_->add_to_stream(c, h);
         stream.invalidate();            // what the gather prepared for the first norm is of the stream before this
+        stream.copy_valid = copied;
     }
     Stream* cur = &stream;
     for (size_t i = 0; i < s.order.size(); ++i) {

@@ -170,6 +170,9 @@ public:
     // steps): it names the need, and is then called with its state's cache entry instead.
     virtual CacheNeed stream_state_need() const { return CacheNeed(); }
     virtual void add_to_stream_with(StepContext& c, Tensor& h, const CacheEntry& state) { (void)state; add_to_stream(c, h); }
+    // Optional: the part also writes the stream's rows in the activation type (for a first block that reads the stream itself).
+    virtual bool writes_stream_copy() const { return false; }
+    virtual void add_to_stream_copy(StepContext& c, Tensor& h, const CacheEntry& state, Tensor& copy) { (void)copy; add_to_stream_with(c, h, state); }
 };
 
 // What a mixer sees of the cache for one run of the order.

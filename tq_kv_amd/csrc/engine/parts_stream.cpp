@@ -55,16 +55,20 @@ public:
         return n;
     }
     void add_to_stream(StepContext&, Tensor&) override { raise(TQE_ERR_STATE, "pair_hash needs its state: the previous token of every sequence"); }
-    void add_to_stream_with(StepContext& c, Tensor& h, const CacheEntry& state) override {
+    void add_to_stream_with(StepContext& c, Tensor& h, const CacheEntry& state) override { add(c, h, state, nullptr); }
+    // the same, and the stream's rows in the activation type where that is bfloat16 (what the first part of a layer reads)
+    void add_to_stream_copy(StepContext& c, Tensor& h, const CacheEntry& state, Tensor& copy) override { add(c, h, state, copy.dtype == BF16 ? copy.data : nullptr); }
+    bool writes_stream_copy() const override { return true; }
+
+private:
+    void add(StepContext& c, Tensor& h, const CacheEntry& state, void* copy) {
         if (state.kind != CacheNeed::State || state.state.dtype != I32) raise(TQE_ERR_STATE, "pair_hash was given no state of the cache");
         int32_t* last = (int32_t*)state.state.data;
         K::pair_embed(table_->t.data, table_->t.dtype, (int)buckets_, mul_prev_, mul_cur_, c.dev.tokens, c.dev.tok_seq, c.dev.tok_pos, c.dev.seq_slot,
-                      c.dev.seq_start, last, (float*)h.data, c.n_tokens, (int)hidden_, (int)vocab_, c.stream);
-        // its own launch: the first token of a sequence's piece reads what the last one writes
-        K::remember_tokens(c.dev.tokens, c.dev.cu, c.dev.seq_new, c.dev.seq_slot, last, c.n_seqs, c.stream);
+                      c.dev.seq_start, last, (float*)h.data, c.n_tokens, (int)hidden_, (int)vocab_, copy, c.all_decode ? 1 : 0, c.stream);
+        // otherwise its own launch: the first token of a sequence's piece reads what the last one writes
+        if (!c.all_decode) K::remember_tokens(c.dev.tokens, c.dev.cu, c.dev.seq_new, c.dev.seq_slot, last, c.n_seqs, c.stream);
     }
-
-private:
     int64_t hidden_, vocab_, buckets_, mul_prev_, mul_cur_;
     std::string tensor_;
     OwnedPtr table_;

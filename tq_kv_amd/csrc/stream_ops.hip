@@ -12,7 +12,8 @@ template <typename TT>
 __global__ __launch_bounds__(256)
 void pair_embed_kernel(const TT* __restrict__ table, int buckets, long long mul_prev, long long mul_cur, const int32_t* __restrict__ tokens,
                        const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ seq_slot,
-                       const int32_t* __restrict__ seq_start, const int32_t* __restrict__ last, float* __restrict__ h, int hidden, int vocab) {
+                       const int32_t* __restrict__ seq_start, int32_t* __restrict__ last, float* __restrict__ h, int hidden, int vocab,
+                       bf16_t* __restrict__ copy, int remember) {
     const int t = blockIdx.x;
     const int pos = tok_pos[t], seq = tok_seq[t];
     const int tok = tokens[t];
@@ -23,9 +24,16 @@ void pair_embed_kernel(const TT* __restrict__ table, int buckets, long long mul_
         row = (prev * mul_prev + (long long)tok * mul_cur) % buckets;
         if (row < 0) row += buckets;
     }
+    // a step of one token a sequence: the token that read the slot's previous token is the one that replaces it
+    __syncthreads();
+    if (remember && threadIdx.x == 0) last[seq_slot[seq]] = tok;
     const TT* src = table + (size_t)row * hidden;
     float* dst = h + (size_t)t * hidden;
-    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] += to_float(src[i]);
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        const float v = dst[i] + to_float(src[i]);
+        dst[i] = v;
+        if (copy) copy[(size_t)t * hidden + i] = from_float<bf16_t>(v);
+    }
 }
 
 // last[slot of sequence s] = the last token the step brings of s
@@ -132,16 +140,16 @@ void row_gate_kernel(const TA* __restrict__ x, const TW* __restrict__ w, float* 
 
 extern "C" int tqk_pair_embed(const void* table, int table_dtype, int buckets, long long mul_prev, long long mul_cur, const int32_t* tokens,
                               const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* seq_slot, const int32_t* seq_start,
-                              const int32_t* last, float* h, int n_tokens, int hidden, int vocab, void* stream) {
+                              int32_t* last, float* h, int n_tokens, int hidden, int vocab, void* copy_bf16, int remember, void* stream) {
     TQK_REQUIRE(table && tokens && tok_seq && tok_pos && seq_slot && seq_start && last && h, "tqk_pair_embed: null pointer");
     TQK_REQUIRE(buckets > 0 && hidden > 0 && n_tokens >= 0 && vocab > 0, "tqk_pair_embed: bad sizes");
     TQK_REQUIRE(mul_prev >= 0 && mul_cur >= 0 && mul_prev < (1LL << 31) && mul_cur < (1LL << 31), "tqk_pair_embed: multipliers out of range");
     if (n_tokens == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     if (table_dtype == TQK_F32)
-        pair_embed_kernel<float><<<n_tokens, 256, 0, s>>>((const float*)table, buckets, mul_prev, mul_cur, tokens, tok_seq, tok_pos, seq_slot, seq_start, last, h, hidden, vocab);
+        pair_embed_kernel<float><<<n_tokens, 256, 0, s>>>((const float*)table, buckets, mul_prev, mul_cur, tokens, tok_seq, tok_pos, seq_slot, seq_start, last, h, hidden, vocab, (bf16_t*)copy_bf16, remember);
     else if (table_dtype == TQK_BF16)
-        pair_embed_kernel<bf16_t><<<n_tokens, 256, 0, s>>>((const bf16_t*)table, buckets, mul_prev, mul_cur, tokens, tok_seq, tok_pos, seq_slot, seq_start, last, h, hidden, vocab);
+        pair_embed_kernel<bf16_t><<<n_tokens, 256, 0, s>>>((const bf16_t*)table, buckets, mul_prev, mul_cur, tokens, tok_seq, tok_pos, seq_slot, seq_start, last, h, hidden, vocab, (bf16_t*)copy_bf16, remember);
     else return tqk_fail("tqk_pair_embed: unknown dtype %d", table_dtype);
     return tqk_check_launch("tqk_pair_embed");
 }

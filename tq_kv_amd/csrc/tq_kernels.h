@@ -264,13 +264,14 @@ int tqk_moe_combine(const void* y, int act_dtype, const int32_t* pair_pos, const
 /* Around the residual stream (stream_ops.hip).  tqk_pair_embed: h[t] += table[(prev * mul_prev + token * mul_cur) mod buckets],
  * table [buckets + 1, hidden], the last row for a sequence's first token; prev is the token before it in the step or, for the
  * first token a step brings of a sequence that has begun, last[slot].  tqk_remember_tokens: last[slot] = the last token the step
- * brings of each sequence (its own launch: the first token of a sequence's piece reads what the last one writes).
+ * brings of each sequence (its own launch: the first token of a sequence's piece reads what the last one writes; in a step of one
+ * token a sequence tqk_pair_embed does it itself, `remember`).  copy_bf16 (or null): the stream's rows after the addition, as bfloat16.
  * tqk_norm_add: h[t] += y[t] / sqrt(mean(y[t]^2) + eps) * weight (weight null: h[t] += y[t]; y null: nothing is added), and
  * copy[t] = h[t] in the activation type (copy may be null).  tqk_unary_act: out = f(x), f a gate's function with u = 1.
  * tqk_row_gate: out[t] = sigmoid(x[t] . w), float32. */
 int tqk_pair_embed(const void* table, int table_dtype, int buckets, long long mul_prev, long long mul_cur, const int32_t* tokens,
                    const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* seq_slot, const int32_t* seq_start,
-                   const int32_t* last, float* h, int n_tokens, int hidden, int vocab, void* stream);
+                   int32_t* last, float* h, int n_tokens, int hidden, int vocab, void* copy_bf16, int remember, void* stream);
 int tqk_remember_tokens(const int32_t* tokens, const int32_t* cu, const int32_t* seq_new, const int32_t* seq_slot, int32_t* last,
                         int n_seqs, void* stream);
 int tqk_norm_add(float* h, const void* y, int act_dtype, const void* weight, int weight_dtype, float eps, void* copy, int n_tokens,

@@ -427,16 +427,38 @@ void attention_masked_block_kernel(const MaskedArgs a) {
 #pragma unroll
         for (int c = 0; c < CT; ++c) {
             float mx = m[c];
+            // three shapes of the same loop, chosen by what holds for the whole wave: most pages of a prompt lie inside what every
+            // column sees and carry no cap, and then a score costs a multiplication and a maximum
+            if (cap > 0.f) {
 #pragma unroll
-            for (int t = 0; t < 4; ++t)
+                for (int t = 0; t < 4; ++t)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int j = key0 + t * 16 + g * 4 + r;
-                    float v = cap > 0.f ? cap2 * tanh_fast(s[c][t][r] * scale_over_cap) : s[c][t][r] * scale2;
-                    if (!inside && !(j <= pos_c[c] && (j >= lo_c[c] || j < kept))) v = -INFINITY;
-                    s[c][t][r] = v;
-                    mx = fmaxf(mx, v);
-                }
+                    for (int r = 0; r < 4; ++r) {
+                        const int j = key0 + t * 16 + g * 4 + r;
+                        float v = cap2 * tanh_fast(s[c][t][r] * scale_over_cap);
+                        if (!inside && !(j <= pos_c[c] && (j >= lo_c[c] || j < kept))) v = -INFINITY;
+                        s[c][t][r] = v;
+                        mx = fmaxf(mx, v);
+                    }
+            } else if (inside) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        s[c][t][r] *= scale2;
+                        mx = fmaxf(mx, s[c][t][r]);
+                    }
+            } else {
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int j = key0 + t * 16 + g * 4 + r;
+                        const float v = (j <= pos_c[c] && (j >= lo_c[c] || j < kept)) ? s[c][t][r] * scale2 : -INFINITY;
+                        s[c][t][r] = v;
+                        mx = fmaxf(mx, v);
+                    }
+            }
             mx = fmaxf(mx, __shfl_xor(mx, 16, TQK_WAVE));
             mx = fmaxf(mx, __shfl_xor(mx, 32, TQK_WAVE));
             const float base = mx == -INFINITY ? 0.f : mx;      // a column that has met no key it sees yet

@@ -83,6 +83,136 @@ void normed_rope_store_kernel(const TA* __restrict__ qkv, const TW* __restrict__
     }
 }
 
+// The same for steps of many tokens in bfloat16 (head sizes multiples of 8, half the rotated elements too), in two launches.
+// Queries and keys: a block per token, a thread per 8 neighbouring elements (16 bytes a load and a store); the sums of squares of a
+// head's pieces meet in LDS; the piece a rotated one turns with is read once more (it is in the caches).
+template <typename TW>
+__global__ __launch_bounds__(256)
+void normed_rope_qk_vec_kernel(const bf16_t* __restrict__ qkv, const TW* __restrict__ q_norm_w, const TW* __restrict__ k_norm_w, float eps,
+                               const float* __restrict__ cos_table, const float* __restrict__ sin_table, int rot_dim, int max_positions,
+                               const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ page_table,
+                               int table_width, bf16_t* __restrict__ keys, bf16_t* __restrict__ q_out, int n_heads, int n_kv_heads, int dk, int dv,
+                               int write_kv) {
+    extern __shared__ float piece_ss[];
+    const int t = blockIdx.x;
+    const int per_head = dk / 8, n_pieces = (n_heads + (write_kv ? n_kv_heads : 0)) * per_head;
+    const size_t total = (size_t)(n_heads + n_kv_heads) * dk + (size_t)n_kv_heads * dv;
+    const bf16_t* row = qkv + (size_t)t * total;
+    auto load8 = [&](const bf16_t* p, float* v) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(p);
+        const uint32_t u[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { v[2 * j] = __uint_as_float(u[j] << 16); v[2 * j + 1] = __uint_as_float(u[j] & 0xffff0000u); }
+    };
+    const bool normed = q_norm_w != nullptr;
+    if (normed) {
+        for (int c = threadIdx.x; c < n_pieces; c += blockDim.x) {
+            float x[8], ss = 0.f;
+            load8(row + (size_t)c * 8, x);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) ss = fmaf(x[j], x[j], ss);
+            piece_ss[c] = ss;
+        }
+        __syncthreads();
+    }
+    const int pos = tok_pos[t];
+    const int half = rot_dim / 2;
+    const bool rotate = rot_dim > 0 && pos < max_positions;
+    int page = -1;
+    if (write_kv) page = page_table[(size_t)tok_seq[t] * table_width + pos / TQK_PAGE];
+    for (int c = threadIdx.x; c < n_pieces; c += blockDim.x) {
+        const int head = c / per_head, off = (c % per_head) * 8;
+        const bool is_q = head < n_heads;
+        if (!is_q && page < 0) continue;                // the host never lets this happen
+        const TW* w = is_q ? q_norm_w : k_norm_w;
+        float inv = 1.f;
+        if (normed) {
+            float ss = 0.f;
+            for (int k = 0; k < per_head; ++k) ss += piece_ss[head * per_head + k];          // the same order for every piece of the head
+            inv = 1.f / sqrtf(ss / (float)dk + eps);
+        }
+        float x[8];
+        load8(row + (size_t)c * 8, x);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) x[j] *= inv * (normed ? to_float(w[off + j]) : 1.f);
+        if (rotate && off < rot_dim) {
+            const bool first = off < half;
+            const int other = first ? off + half : off - half, p = first ? off : off - half;
+            float y[8];
+            load8(row + (size_t)head * dk + other, y);
+            // (half and p are multiples of 8: the eight angles of a piece are two aligned loads of 16 bytes from each table)
+            const float4* ct = reinterpret_cast<const float4*>(cos_table + (size_t)pos * half + p);
+            const float4* st = reinterpret_cast<const float4*>(sin_table + (size_t)pos * half + p);
+            const float4 c0 = ct[0], c1 = ct[1], s0 = st[0], s1 = st[1];
+            const float cs[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w}, sn[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float yn = y[j] * inv * (normed ? to_float(w[other + j]) : 1.f);
+                x[j] = first ? x[j] * cs[j] - yn * sn[j] : x[j] * cs[j] + yn * sn[j];
+            }
+        }
+        uint4 out;
+        out.x = float_to_bf16_bits(x[0]) | ((uint32_t)float_to_bf16_bits(x[1]) << 16);
+        out.y = float_to_bf16_bits(x[2]) | ((uint32_t)float_to_bf16_bits(x[3]) << 16);
+        out.z = float_to_bf16_bits(x[4]) | ((uint32_t)float_to_bf16_bits(x[5]) << 16);
+        out.w = float_to_bf16_bits(x[6]) | ((uint32_t)float_to_bf16_bits(x[7]) << 16);
+        bf16_t* dst = is_q ? q_out + ((size_t)t * n_heads + head) * dk + off
+                           : keys + (((size_t)page * n_kv_heads + (head - n_heads)) * TQK_PAGE + pos % TQK_PAGE) * dk + off;
+        *reinterpret_cast<uint4*>(dst) = out;
+    }
+}
+
+// Values: the cache keeps them transposed inside a page, so here the lanes run along the tokens (64 a block, one kv head, the waves
+// taking pieces of 8 elements in turn): where the tokens are neighbours in a sequence, a wave's stores of one element fall into one row
+// of 128 bytes.  Every lane finds its own page and place, so nothing depends on the tokens being neighbours.
+template <typename TW>
+__global__ __launch_bounds__(256)
+void mixed_values_store_vec_kernel(const bf16_t* __restrict__ qkv, const TW* __restrict__ mix, const bf16_t* __restrict__ mix_with,
+                                   bf16_t* __restrict__ mix_keep, const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos,
+                                   const int32_t* __restrict__ page_table, int table_width, bf16_t* __restrict__ values, int n_tokens, int n_heads,
+                                   int n_kv_heads, int dk, int dv) {
+    const int lane = threadIdx.x % TQK_WAVE, wave = threadIdx.x / TQK_WAVE, n_waves = blockDim.x / TQK_WAVE;
+    const int t = (blockIdx.x / n_kv_heads) * TQK_WAVE + lane, g = blockIdx.x % n_kv_heads;
+    if (t >= n_tokens) return;
+    const int pos = tok_pos[t];
+    const int page = page_table[(size_t)tok_seq[t] * table_width + pos / TQK_PAGE];
+    if (page < 0) return;                               // the host never lets this happen
+    bf16_t* dst = values + ((size_t)page * n_kv_heads + g) * TQK_PAGE * dv + value_place(pos % TQK_PAGE);
+    const size_t total = (size_t)(n_heads + n_kv_heads) * dk + (size_t)n_kv_heads * dv;
+    const bf16_t* src = qkv + (size_t)t * total + (size_t)(n_heads + n_kv_heads) * dk + (size_t)g * dv;
+    const float lam = mix && mix_with ? to_float(mix[0]) : 0.f;
+    for (int c = wave * 8; c < dv; c += n_waves * 8) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(src + c);
+        const uint32_t u[4] = {raw.x, raw.y, raw.z, raw.w};
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { v[2 * j] = __uint_as_float(u[j] << 16); v[2 * j + 1] = __uint_as_float(u[j] & 0xffff0000u); }
+        const size_t at = ((size_t)t * n_kv_heads + g) * dv + c;
+        if (mix_with) {
+            const uint4 mr = *reinterpret_cast<const uint4*>(mix_with + at);
+            const uint32_t mu[4] = {mr.x, mr.y, mr.z, mr.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                v[2 * j] = (1.f - lam) * v[2 * j] + lam * __uint_as_float(mu[j] << 16);
+                v[2 * j + 1] = (1.f - lam) * v[2 * j + 1] + lam * __uint_as_float(mu[j] & 0xffff0000u);
+            }
+        }
+        uint16_t bits[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) bits[j] = float_to_bf16_bits(v[j]);
+        if (mix_keep) {
+            uint4 out;
+            out.x = bits[0] | ((uint32_t)bits[1] << 16);
+            out.y = bits[2] | ((uint32_t)bits[3] << 16);
+            out.z = bits[4] | ((uint32_t)bits[5] << 16);
+            out.w = bits[6] | ((uint32_t)bits[7] << 16);
+            *reinterpret_cast<uint4*>(mix_keep + at) = out;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) dst[(size_t)(c + j) * TQK_PAGE].bits = bits[j];
+    }
+}
+
 // ---- attention, a wave per (token, head) --------------------------------------------------------------
 // Keys are taken a page at a time; lane j computes the score of key j of the page, the softmax runs online over the
 // pages, then lane c accumulates output element c (+64, ...).  The order of operations for a query depends on its
@@ -175,6 +305,22 @@ extern "C" int tqk_normed_rope_store(const void* qkv, int act_dtype, const void*
     TQK_REQUIRE(!mix_with || mix, "tqk_normed_rope_store: values to mix with, but no weight");
     if (n_tokens == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
+    // steps of many tokens in bfloat16 whose sizes fall into pieces of 16 bytes: the two launches above
+    const long long pieces = (long long)(n_heads + n_kv_heads) * key_dim / 8;
+    if (act_dtype == TQK_BF16 && n_tokens > 64 && key_dim % 8 == 0 && value_dim % 8 == 0 && rot_dim % 16 == 0 && pieces <= 8192 &&
+        (!q_norm_w) == (!k_norm_w)) {
+        const size_t lds = (size_t)pieces * sizeof(float);
+        const long long v_blocks = (long long)((n_tokens + TQK_WAVE - 1) / TQK_WAVE) * n_kv_heads;
+        TQK_REQUIRE(v_blocks <= 0x7fffffff, "tqk_normed_rope_store: too many tokens");
+#define TQK_NRV(TW) \
+        normed_rope_qk_vec_kernel<TW><<<n_tokens, 256, lds, s>>>((const bf16_t*)qkv, (const TW*)q_norm_w, (const TW*)k_norm_w, eps, cos_table, sin_table, rot_dim, \
+            max_positions, tok_seq, tok_pos, page_table, table_width, (bf16_t*)keys, (bf16_t*)q_out, n_heads, n_kv_heads, key_dim, value_dim, write_kv); \
+        if (write_kv) mixed_values_store_vec_kernel<TW><<<(unsigned)v_blocks, 256, 0, s>>>((const bf16_t*)qkv, (const TW*)mix, (const bf16_t*)mix_with, \
+            (bf16_t*)mix_keep, tok_seq, tok_pos, page_table, table_width, (bf16_t*)values, n_tokens, n_heads, n_kv_heads, key_dim, value_dim)
+        if (w_dtype == TQK_F32) { TQK_NRV(float); } else if (w_dtype == TQK_BF16) { TQK_NRV(bf16_t); } else return tqk_fail("tqk_normed_rope_store: unknown dtype %d", w_dtype);
+#undef TQK_NRV
+        return tqk_check_launch("tqk_normed_rope_store");
+    }
     dim3 grid(n_tokens, (n_heads + 2 * n_kv_heads + AM_WAVES - 1) / AM_WAVES);
 #define TQK_NRS(TA, TW) \
     normed_rope_store_kernel<TA, TW><<<grid, AM_WAVES * TQK_WAVE, 0, s>>>((const TA*)qkv, (const TW*)q_norm_w, (const TW*)k_norm_w, eps, cos_table, sin_table, \

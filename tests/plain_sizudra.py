@@ -131,15 +131,22 @@ def expert(x, w, p, low):
     return product(torch.relu(u) ** 2, w[p + "down"], low)
 
 
-def route(x, w_router, top, low):
-    """The `top` experts with the largest logits (float32), and the softmax over those logits alone."""
+def route(x, w_router, top, low, margins=None):
+    """The `top` experts with the largest logits (float32), and the softmax over those logits alone.  margins (a list, optional) gets,
+    per token, how far the last chosen logit lies above the first one left out, in units of the logits' spread (inf where all are chosen)."""
     z = rnd(x, low) @ w_router.T
     val, idx = torch.topk(z, top, dim=-1)
+    if margins is not None:
+        if top < z.shape[-1]:
+            ordered = z.sort(-1, descending=True).values
+            margins.append((ordered[:, top - 1] - ordered[:, top]) / z.std(-1).clamp_min(1e-6))
+        else:
+            margins.append(torch.full((z.shape[0],), float("inf")))
     return idx, torch.softmax(val, dim=-1)
 
 
-def moe_ff(x, w, p, f, low):
-    idx, wt = route(x, w[p + "router"], f["router"]["top"], low)
+def moe_ff(x, w, p, f, low, margins=None):
+    idx, wt = route(x, w[p + "router"], f["router"]["top"], low, margins)
     out = torch.zeros_like(x)
     for t in range(x.shape[0]):
         for c in range(idx.shape[1]):
@@ -150,8 +157,8 @@ def moe_ff(x, w, p, f, low):
     return out
 
 
-def forward(cfg, w, tokens, low=F32, layers_out=None):
-    """Logits [T, vocab] of one sequence from its first token."""
+def forward(cfg, w, tokens, low=F32, layers_out=None, margins=None):
+    """Logits [T, vocab] of one sequence from its first token.  margins: see route (one entry per layer of experts)."""
     tokens = torch.as_tensor(tokens, dtype=torch.long)
     eps = cfg["norm"]["eps"]
     big = cfg["embedding"]["bigram"]
@@ -163,7 +170,7 @@ def forward(cfg, w, tokens, low=F32, layers_out=None):
         x = x + rms_norm(mixer(x, w, p + "mix.", layer["mixer"], eps, positions, low, carried), w[p + "norm1"], eps)
         f = layer.get("mlp")
         if f:
-            y = dense_ff(x, w, p + "mlp.", low) if f["kind"] == "dense" else moe_ff(x, w, p + "mlp.", f, low)
+            y = dense_ff(x, w, p + "mlp.", low) if f["kind"] == "dense" else moe_ff(x, w, p + "mlp.", f, low, margins)
             x = x + rms_norm(y, w[p + "norm2"], eps)
         if layers_out is not None:
             layers_out.append(x.clone())

@@ -159,5 +159,30 @@ def close(got, want, dtype, what="", spare=0.03):
     assert over <= max(1, int(spare * e.numel())) and e.max().item() < 1.5, "%s: %d of %d rows over, worst %.3g" % (what, over, e.numel(), e.max().item())
 
 
+def close_typical(got, want, dtype, what=""):
+    """For models drawn at random, some of them small and with several layers of experts, where bfloat16 rounding moves a router's
+    choice now and then and the moved token is seen by later ones: float32 as `close`; bfloat16 by the typical row (the median within
+    0.08 of the spread, no more than an eighth of the rows beyond 0.15, none beyond 1.5).  A fault of structure (a head read from the
+    wrong group, a window one off, a sink left out) moves every row."""
+    if dtype == "float32":
+        return close(got, want, dtype, what)
+    assert got.shape == want.shape, "%s: shapes %s and %s" % (what, tuple(got.shape), tuple(want.shape))
+    e = row_errors(got.reshape(-1, got.shape[-1]), want.reshape(-1, want.shape[-1]))
+    assert torch.isfinite(e).all(), "%s: logits are not finite" % what
+    over = (e > 0.15).float().mean().item()
+    assert e.median().item() <= 0.08 and over <= 0.125 and e.max().item() < 1.5, "%s: median %.3g, %.3g of the rows over, worst %.3g" % (
+        what, e.median().item(), over, e.max().item())
+
+
 def plain_logits(cfg, w, toks, low=torch.float32):
     return plain.forward(cfg, as_float(w), toks, low)
+
+
+def sure_rows(cfg, w, toks, least=0.1):
+    """Which rows' routers all choose by a margin that rounding to bfloat16 does not reach (in units of the logits' spread)."""
+    margins = []
+    plain.forward(cfg, as_float(w), toks, margins=margins)
+    sure = torch.ones(len(toks), dtype=torch.bool)
+    for m in margins:
+        sure &= m > least
+    return sure

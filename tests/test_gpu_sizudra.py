@@ -440,3 +440,15 @@ def test_replay_of_steps_and_the_command_line(dtype, tmp_path_factory):
     for t in tokens:
         assert int(S.plain_logits(cfg, w, seq)[-1].argmax()) == t
         seq.append(t)
+
+
+def test_a_model_of_more_windows_than_the_cache_has_groups(tmp_path_factory):
+    """Twenty layers with twenty windows: the cache keeps every page in one group, and each layer still sees its own window."""
+    cfg = S.config(50, 32, [(S.mixer(2, 1, 8, 8, 4, v_mix=l % 3 == 0, window=3 + 4 * l, keep_first=l % 5), S.dense(24) if l % 2 else None) for l in range(20)])
+    w = S.weights(cfg, seed=5)
+    eng = Engine(Model.from_dir(S.write_folder(str(tmp_path_factory.mktemp("sizudra_windows")), cfg, w), dtype="float32"), max_tokens=64 * 8, max_slots=2)
+    assert len(eng.cache.kv_groups) == 1
+    toks = S.tokens(150, cfg["vocab"], 9)
+    want = S.plain_logits(cfg, w, toks)
+    S.close(run_cut(eng, toks, []), want, "float32", "whole")
+    S.close(run_cut(eng, toks, [70] + list(range(100, 150))), want, "float32", "a portion and single tokens")

@@ -145,3 +145,14 @@ def test_plain_rotation_turns_the_first_elements_only():
 def test_plain_router_renormalises_over_the_chosen():
     idx, wt = plain.route(torch.tensor([[1.0, 0.0]]), torch.tensor([[2.0, 0.0], [0.0, 1.0], [1.0, 0.0], [-1.0, 0.0]]), 2, torch.float32)
     assert idx.tolist() == [[0, 2]] and torch.allclose(wt, torch.softmax(torch.tensor([[2.0, 1.0]]), -1))
+
+
+def test_more_windows_than_the_cache_has_groups_keep_every_page():
+    a = [(S.mixer(2, 1, 8, 8, 4, window=3 + i, keep_first=1), None) for i in range(20)]
+    spec = spec_from_dict(S.config(50, 16, a))
+    assert all(l.block.params["mixer"].params["cache_keeps_all"] for l in spec.layers)
+    model = Model(spec, dtype="float32", device="cpu")
+    assert len({(n.window, n.keep_first) for n in model.needs[:20]}) == 1 and model.needs[0].window is None
+    few = spec_from_dict(S.config(50, 16, a[:5]))
+    assert not any(l.block.params["mixer"].params["cache_keeps_all"] for l in few.layers)
+    assert [n.window for n in Model(few, dtype="float32", device="cpu").needs[:5]] == [3, 4, 5, 6, 7]

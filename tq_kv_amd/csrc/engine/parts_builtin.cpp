@@ -238,7 +238,8 @@ public:
 // window: a sequence's first positions stay visible, at their true places); sink (a learned number per head whose
 // exponential joins the softmax's denominator, with no key and no value); value_mix "source" (the values of the
 // step's tokens are handed to later layers) or "mixed" (v <- (1 - lambda) v + lambda v_source with a learned scalar,
-// before the cache); value_mix_key (which source, "values" unless given); names: the tensors' names inside the
+// before the cache); value_mix_key (which source, "values" unless given); cache_keeps_all (the cache keeps every page although the
+// mixer sees a window); names: the tensors' names inside the
 // part's prefix {q, k, v, o, q_norm, k_norm, sink, mix}.  With any of them the step runs through the kernels of
 // attention_masked.hip.
 //
@@ -267,6 +268,7 @@ public:
         eps_ = qk_norm_ ? (float)r.number("eps") : 0.f;
         cap_ = r.has("cap") ? (float)r.number("cap", true) : 0.f;
         keep_first_ = (int)r.integer_or("keep_first", 0, 0);
+        cache_keeps_all_ = r.boolean_or("cache_keeps_all", false);
         has_sink_ = r.boolean_or("sink", false);
         const std::string mixing = r.string_or("value_mix", "none");
         if (mixing == "none") value_mix_ = MIX_NONE;
@@ -365,8 +367,10 @@ public:
         n.kind = CacheNeed::Pages;
         n.key_page = {n_kv_heads_, TQE_PAGE, head_dim_};
         n.value_page = {n_kv_heads_, value_dim_, TQE_PAGE};
-        n.window = window_;
-        n.keep_first = keep_first_;
+        // (cache_keeps_all: the cache gives no page back although the mixer sees a window, so that layers of many different windows
+        // can share one group of the cache)
+        n.window = cache_keeps_all_ ? 0 : window_;
+        n.keep_first = cache_keeps_all_ ? 0 : keep_first_;
         return n;
     }
 
@@ -641,7 +645,7 @@ private:
     float scale_;
     enum { MIX_NONE = 0, MIX_SOURCE = 1, MIX_MIXED = 2 };
     int value_dim_, keep_first_, value_mix_ = MIX_NONE;
-    bool qk_norm_ = false, has_sink_ = false, extras_ = false;
+    bool qk_norm_ = false, has_sink_ = false, extras_ = false, cache_keeps_all_ = false;
     float eps_ = 0.f, cap_ = 0.f;
     std::string mix_key_, n_q_, n_k_, n_v_, n_o_, n_q_norm_, n_k_norm_, n_sink_, n_mix_;
     std::shared_ptr<Position> position_;

@@ -56,6 +56,7 @@ Json mixer_typed(const Json& raw, const std::string& where, bool second) {
         KeyReader mask(object_at(raw, "mask", where), where + ".mask");
         m.set("window", mask.integer("size", 1));
         m.set("keep_first", mask.integer_or("keep_first", 0, 0));
+        if (m["window"].as_int() > 0x3fffffff || m["keep_first"].as_int() > 0x3fffffff) raise(TQE_ERR_CONFIG, "%s.mask: size or keep_first is out of range", where.c_str());
     } else {
         m.set("softcap", Json());
         m.set("window", Json());
@@ -151,6 +152,16 @@ ModelSpec sizudra_spec(const Json& c) {
     s.stream_position = part("pair_hash", {{"hidden", width}, {"vocab", c["vocab"]}, {"buckets", c["bigram_buckets"]}, {"mul_prev", c["bigram_mul_prev"]},
                                            {"mul_cur", c["bigram_mul_cur"]}, {"max_positions", c["max_positions"]}, {"tensor", ""}});
     s.stream_position_prefix = "bigram";
+    // Layers of equal head sizes and equal windows share a group of the cache, and the cache's bookkeeping takes TQE_MAX_GROUPS of
+    // them: a model with more different windows than that keeps every page (what a layer sees is its own window still).
+    std::vector<std::vector<long long>> distinct;
+    for (const Json& layer : c["layers"].items()) {
+        const Json& m = layer["mixer"];
+        const std::vector<long long> key = {m["kv_heads"].as_int(), m["dim"].as_int(), m["vdim"].as_int(), m["window"].is_null() ? 0 : m["window"].as_int(),
+                                            m["keep_first"].as_int()};
+        if (std::find(distinct.begin(), distinct.end(), key) == distinct.end()) distinct.push_back(key);
+    }
+    const bool keep_all = (int)distinct.size() > TQE_MAX_GROUPS;
     bool mixing_begun = false;
     size_t l = 0;
     for (const Json& layer : c["layers"].items()) {
@@ -164,7 +175,7 @@ ModelSpec sizudra_spec(const Json& c) {
         if (m["v_mix"].as_bool()) mixing_begun = true;
         const PartSpec mixer = part("attention", {{"hidden", width}, {"n_heads", m["heads"]}, {"n_kv_heads", m["kv_heads"]}, {"head_dim", m["dim"]},
                                                   {"value_dim", m["vdim"]}, {"scale", m["scale"]}, {"qk_norm", true}, {"eps", c["norm_eps"]},
-                                                  {"window", m["window"]}, {"keep_first", m["keep_first"]}, {"cap", m["softcap"]}, {"sink", second},
+                                                  {"window", m["window"]}, {"keep_first", m["keep_first"]}, {"cache_keeps_all", keep_all}, {"cap", m["softcap"]}, {"sink", second},
                                                   {"value_mix", value_mix}, {"position", position.to_json()},
                                                   {"names", names_of({{"q", "q"}, {"k", "k"}, {"v", "v"}, {"o", "o"}, {"q_norm", "q.norm"}, {"k_norm", "k.norm"},
                                                                       {"sink", "sink"}, {"mix", "vmix"}})}});

@@ -290,18 +290,19 @@ void attention_masked_mfma_kernel(const MaskedArgs a) {
     }
 }
 
-// Tiles, with a page staged once for a block.  A block of four waves takes one kv head and a tile of consecutive queries
-// of one sequence: its waves are min(4, heads of the group) query heads times 4 / that many sub-tiles of 16 CT queries
-// (CT = 2; a group of one head: 128 queries a block; of two: 64; of four or more: 32, the further heads in further
-// blocks).  A wave holds CT sets of 16 columns, so that what it reads of a page from LDS serves CT products.  Every
+// Tiles, with a page staged once for a block.  A block of W = 4 or 8 waves takes one kv head and a tile of consecutive queries
+// of one sequence: its waves are min(4, heads of the group) query heads times W / that many sub-tiles of 16 CT queries
+// (CT = 2; with four waves a group of one head: 128 queries a block; of two: 64; of four or more: 32, the further heads in
+// further blocks; with eight waves twice that, for steps that give blocks enough).  A wave holds CT sets of 16 columns, so that what it reads of a page from LDS serves CT products.  Every
 // thread brings its pieces of the next page's keys and values into registers while the block computes on the page that
 // lies in LDS (two pages under way were measured no faster; rows padded by 16 bytes, so that the 16 rows a load of the matrix cores' operands touches fall on
 // different banks); a wave passes over a page none of its queries sees.  Sizes up to 128 and 128.
-template <int KB, int DB, int CT>
-__global__ __launch_bounds__(4 * TQK_WAVE) __attribute__((amdgpu_waves_per_eu(2, 2)))
+template <int KB, int DB, int CT, int W>
+__global__ __launch_bounds__(W * TQK_WAVE) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void attention_masked_block_kernel(const MaskedArgs a) {
     constexpr int KS_MAX = KB * 64 + 16, VS = 2 * TQK_PAGE + 16;        // bytes of a key row and of a value row in LDS
-    constexpr int VJ = (DB + 1) / 2;                                        // pieces of values a thread brings
+    constexpr int THREADS = W * TQK_WAVE;
+    constexpr int KJ = (KB * 256 + THREADS - 1) / THREADS, VJ = (DB * 128 + THREADS - 1) / THREADS;     // pieces of keys and of values a thread brings
     constexpr int SUB = 16 * CT;                                            // queries of a wave
     __shared__ __attribute__((aligned(16))) unsigned char lds_k[TQK_PAGE * KS_MAX];
     __shared__ __attribute__((aligned(16))) unsigned char lds_v[DB * 16 * VS];
@@ -309,7 +310,7 @@ void attention_masked_block_kernel(const MaskedArgs a) {
     const int col = lane % 16, g = lane / 16;
     const int n_rep = a.n_heads / a.n_kv_heads;
     const int dk = a.dk, dv = a.dv, ks = dk * 2 + 16;
-    const int hpb = min(n_rep, 4), sph = 4 / hpb, chunks = (n_rep + hpb - 1) / hpb;
+    const int hpb = min(n_rep, 4), sph = W / hpb, chunks = (n_rep + hpb - 1) / hpb;
     const int kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
     const int tile = blockIdx.x;
     const int seq = a.tile_seq[tile], tok0 = a.tile_tok0[tile], count = a.tile_count[tile];
@@ -345,18 +346,18 @@ void attention_masked_block_kernel(const MaskedArgs a) {
     const int n_visits = kept_pages + last_page - first_win_page + 1;
 
     // where the thread's pieces of a page (16 bytes each) come from and go to
-    int k_src[KB], k_dst[KB], v_src[VJ], v_dst[VJ];
+    int k_src[KJ], k_dst[KJ], v_src[VJ], v_dst[VJ];
     const int k_per_row = dk / 8;
 #pragma unroll
-    for (int j = 0; j < KB; ++j) {
-        const int p = tid + 256 * j;
+    for (int j = 0; j < KJ; ++j) {
+        const int p = tid + THREADS * j;
         const int pk = p < 8 * dk ? p : tid % (8 * dk);       // a piece beyond the page: one that is there, once more (the same bytes to the same place)
         k_src[j] = pk;
         k_dst[j] = (pk / k_per_row) * ks + (pk % k_per_row) * 16;
     }
 #pragma unroll
     for (int j = 0; j < VJ; ++j) {
-        const int p = tid + 256 * j;
+        const int p = tid + THREADS * j;
         const int pv = p < 8 * dv ? p : tid % (8 * dv);
         v_src[j] = pv;
         v_dst[j] = (pv / 8) * VS + (pv % 8) * 16;
@@ -380,14 +381,14 @@ void attention_masked_block_kernel(const MaskedArgs a) {
     const int32_t* pages = a.page_table + (size_t)seq * a.table_width;
     const size_t k_stride = (size_t)a.n_kv_heads * TQK_PAGE * dk, v_stride = (size_t)a.n_kv_heads * TQK_PAGE * dv;
     auto page_of = [&](int visit) { return visit < kept_pages ? visit : first_win_page + (visit - kept_pages); };
-    uint4 k_reg[KB], v_reg[VJ];
+    uint4 k_reg[KJ], v_reg[VJ];
     auto fetch = [&](int visit) {
         const int page = __builtin_amdgcn_readfirstlane(pages[page_of(visit)]);
         if (page < 0) return;                           // nothing of it is visible to anyone: what LDS then holds is not looked at
         const uint4* kp = reinterpret_cast<const uint4*>(a.keys + (size_t)page * k_stride + (size_t)kvh * TQK_PAGE * dk);
         const uint4* vp = reinterpret_cast<const uint4*>(a.values + (size_t)page * v_stride + (size_t)kvh * TQK_PAGE * dv);
 #pragma unroll
-        for (int j = 0; j < KB; ++j) k_reg[j] = kp[k_src[j]];
+        for (int j = 0; j < KJ; ++j) k_reg[j] = kp[k_src[j]];
 #pragma unroll
         for (int j = 0; j < VJ; ++j) v_reg[j] = vp[v_src[j]];
     };
@@ -397,7 +398,7 @@ void attention_masked_block_kernel(const MaskedArgs a) {
         const int page = __builtin_amdgcn_readfirstlane(pages[pg]);
         __syncthreads();                                // everyone has done with the page before
 #pragma unroll
-        for (int j = 0; j < KB; ++j) *reinterpret_cast<uint4*>(lds_k + k_dst[j]) = k_reg[j];
+        for (int j = 0; j < KJ; ++j) *reinterpret_cast<uint4*>(lds_k + k_dst[j]) = k_reg[j];
 #pragma unroll
         for (int j = 0; j < VJ; ++j) *reinterpret_cast<uint4*>(lds_v + v_dst[j]) = v_reg[j];
         __syncthreads();
@@ -539,12 +540,14 @@ __global__ void attention_masked_merge_kernel(const float* __restrict__ part_out
 }
 
 template <int KB, int DB>
-int launch_masked(const MaskedArgs& a, bool tiles, int n_tiles, int n_rows, hipStream_t s) {
+int launch_masked(const MaskedArgs& a, bool tiles, int n_tiles, int tile_queries, int n_rows, hipStream_t s) {
     if (tiles) {
         if constexpr (KB <= 4 && DB <= 8) {
             const int n_rep = a.n_heads / a.n_kv_heads, hpb = n_rep < 4 ? n_rep : 4;
             dim3 grid(n_tiles, a.n_kv_heads * ((n_rep + hpb - 1) / hpb));
-            attention_masked_block_kernel<KB, DB, 2><<<grid, 4 * TQK_WAVE, 0, s>>>(a);
+            // eight waves a block where the tiles are that large: a page brought in then serves twice the queries
+            if (tile_queries >= 32 * (8 / hpb)) attention_masked_block_kernel<KB, DB, 2, 8><<<grid, 8 * TQK_WAVE, 0, s>>>(a);
+            else attention_masked_block_kernel<KB, DB, 2, 4><<<grid, 4 * TQK_WAVE, 0, s>>>(a);
         } else {
             dim3 grid(n_tiles, (a.n_heads + 3) / 4);
             attention_masked_mfma_kernel<KB, DB, 4, true><<<grid, 4 * TQK_WAVE, 0, s>>>(a);
@@ -559,11 +562,11 @@ int launch_masked(const MaskedArgs& a, bool tiles, int n_tiles, int n_rows, hipS
 }
 
 template <int KB>
-int launch_masked_dv(const MaskedArgs& a, bool tiles, int n_tiles, int n_rows, hipStream_t s) {
-    if (a.dv <= 32) return launch_masked<KB, 2>(a, tiles, n_tiles, n_rows, s);
-    if (a.dv <= 64) return launch_masked<KB, 4>(a, tiles, n_tiles, n_rows, s);
-    if (a.dv <= 128) return launch_masked<KB, 8>(a, tiles, n_tiles, n_rows, s);
-    return launch_masked<KB, 16>(a, tiles, n_tiles, n_rows, s);
+int launch_masked_dv(const MaskedArgs& a, bool tiles, int n_tiles, int tile_queries, int n_rows, hipStream_t s) {
+    if (a.dv <= 32) return launch_masked<KB, 2>(a, tiles, n_tiles, tile_queries, n_rows, s);
+    if (a.dv <= 64) return launch_masked<KB, 4>(a, tiles, n_tiles, tile_queries, n_rows, s);
+    if (a.dv <= 128) return launch_masked<KB, 8>(a, tiles, n_tiles, tile_queries, n_rows, s);
+    return launch_masked<KB, 16>(a, tiles, n_tiles, tile_queries, n_rows, s);
 }
 
 }  // namespace
@@ -572,10 +575,12 @@ extern "C" int tqk_attention_masked_mfma_supported(int key_dim, int value_dim) {
     return key_dim > 0 && key_dim % 8 == 0 && key_dim <= 256 && value_dim > 0 && value_dim <= 256;
 }
 /* queries per tile for steps of several tokens a sequence: 32 for each sub-tile a block's waves make of a tile */
-extern "C" int tqk_attention_masked_mfma_tile(int n_heads, int n_kv_heads, int key_dim, int value_dim) {
+extern "C" int tqk_attention_masked_mfma_tile(int n_tokens, int n_heads, int n_kv_heads, int key_dim, int value_dim) {
     if (key_dim > 128 || value_dim > 128 || n_kv_heads <= 0) return 16;
-    const int n_rep = n_heads / n_kv_heads;
-    return 32 * (4 / (n_rep < 4 ? (n_rep > 0 ? n_rep : 1) : 4));
+    const int n_rep = n_heads / n_kv_heads, hpb = n_rep < 4 ? (n_rep > 0 ? n_rep : 1) : 4;
+    // blocks of four waves, or of eight (twice the queries for every page brought in) where that still leaves four blocks a compute unit
+    const long long blocks8 = (long long)((n_tokens + 32 * (8 / hpb) - 1) / (32 * (8 / hpb))) * n_kv_heads * ((n_rep + hpb - 1) / hpb);
+    return 32 * ((blocks8 >= 1024 ? 8 : 4) / hpb);
 }
 
 /* n_tiles > 0: tiles of up to 16 consecutive queries of one sequence (tile_seq, tile_tok0, tile_count on the device; tok_pos and q by
@@ -585,7 +590,7 @@ extern "C" int tqk_attention_masked_mfma_tile(int n_heads, int n_kv_heads, int k
 extern "C" int tqk_attention_masked_mfma(const void* q, const void* keys, const void* values, const int32_t* tok_pos, const int32_t* page_table,
                                          int table_width, int n_pages, int window, int keep_first, float scale, float cap, const void* sink,
                                          int sink_dtype, const int32_t* tile_seq, const int32_t* tile_tok0, const int32_t* tile_count, int n_tiles,
-                                         int n_rows, int n_parts, void* part_out, void* part_ml, void* out, int n_heads, int n_kv_heads,
+                                         int tile_queries, int n_rows, int n_parts, void* part_out, void* part_ml, void* out, int n_heads, int n_kv_heads,
                                          int key_dim, int value_dim, void* stream) {
     TQK_REQUIRE(q && keys && values && tok_pos && page_table && out, "tqk_attention_masked_mfma: null pointer");
     TQK_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0, "tqk_attention_masked_mfma: %d heads and %d kv heads", n_heads, n_kv_heads);
@@ -594,7 +599,7 @@ extern "C" int tqk_attention_masked_mfma(const void* q, const void* keys, const 
     TQK_REQUIRE(window >= 0 && keep_first >= 0 && cap >= 0.f, "tqk_attention_masked_mfma: negative window, kept positions or cap");
     TQK_REQUIRE(!sink || sink_dtype == TQK_F32 || sink_dtype == TQK_BF16, "tqk_attention_masked_mfma: unknown dtype %d of the sink", sink_dtype);
     const bool tiles = n_tiles > 0;
-    if (tiles) TQK_REQUIRE(tile_seq && tile_tok0 && tile_count && n_tiles <= 0x7fffffff, "tqk_attention_masked_mfma: tiles without their lists");
+    if (tiles) TQK_REQUIRE(tile_seq && tile_tok0 && tile_count && tile_queries >= 16, "tqk_attention_masked_mfma: tiles without their lists or their size");
     else {
         TQK_REQUIRE(n_rows >= 0 && n_rows <= 65535, "tqk_attention_masked_mfma: %d rows", n_rows);
         TQK_REQUIRE(n_parts > 0 && n_parts <= 65535 && (n_parts == 1 || (part_out && part_ml)), "tqk_attention_masked_mfma: %d partitions, or no room for them", n_parts);
@@ -613,9 +618,9 @@ extern "C" int tqk_attention_masked_mfma(const void* q, const void* keys, const 
     a.part_out = (float*)part_out; a.part_ml = (float*)part_ml; a.out = (bf16_t*)out;
     hipStream_t s = (hipStream_t)stream;
     int status;
-    if (key_dim <= 64) status = launch_masked_dv<2>(a, tiles, n_tiles, n_rows, s);
-    else if (key_dim <= 128) status = launch_masked_dv<4>(a, tiles, n_tiles, n_rows, s);
-    else status = launch_masked_dv<8>(a, tiles, n_tiles, n_rows, s);
+    if (key_dim <= 64) status = launch_masked_dv<2>(a, tiles, n_tiles, tile_queries, n_rows, s);
+    else if (key_dim <= 128) status = launch_masked_dv<4>(a, tiles, n_tiles, tile_queries, n_rows, s);
+    else status = launch_masked_dv<8>(a, tiles, n_tiles, tile_queries, n_rows, s);
     if (status || tiles || n_parts == 1) return status;
     attention_masked_merge_kernel<<<n_rows * n_heads, value_dim >= 128 ? 128 : 64, 0, s>>>((const float*)part_out, (const float*)part_ml, n_parts, value_dim,
                                                                                             n_heads, sink, a.sink_f32, (bf16_t*)out);

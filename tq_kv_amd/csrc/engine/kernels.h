@@ -80,8 +80,8 @@ TQ_KERNEL(normed_rope_store, cptr, int, cptr, cptr, int, float, cf32, cf32, int,
           int, int, int, int, int, int, void*);
 TQ_QUERY(int, attention_masked_max_dim);
 TQ_QUERY(int, attention_masked_mfma_supported, int, int);
-TQ_QUERY(int, attention_masked_mfma_tile, int, int, int, int);
-TQ_KERNEL(attention_masked_mfma, cptr, cptr, cptr, ci32, ci32, int, int, int, int, float, float, cptr, int, ci32, ci32, ci32, int, int, int, void*, void*,
+TQ_QUERY(int, attention_masked_mfma_tile, int, int, int, int, int);
+TQ_KERNEL(attention_masked_mfma, cptr, cptr, cptr, ci32, ci32, int, int, int, int, float, float, cptr, int, ci32, ci32, ci32, int, int, int, int, void*, void*,
           void*, int, int, int, int, void*);
 TQ_KERNEL(attention_masked, cptr, cptr, cptr, int, ci32, ci32, ci32, int, int, int, int, int, float, float, cptr, int, void*, int, int, int, int,
           int, void*);

@@ -486,15 +486,15 @@ private:
                     part_ml = c.alloc(F32, {n, n_heads_, n_parts, 2});
                 }
                 K::attention_masked_mfma(q.data, entry.keys.data, entry.values.data, tok_pos, row_table, table.width, n_pages, window_, keep_first_, scale_,
-                                         cap_, sink, sink_dtype, nullptr, nullptr, nullptr, 0, n, n_parts, part_out.data, part_ml.data, out.data, n_heads_,
+                                         cap_, sink, sink_dtype, nullptr, nullptr, nullptr, 0, 0, n, n_parts, part_out.data, part_ml.data, out.data, n_heads_,
                                          n_kv_heads_, head_dim_, value_dim_, c.stream);
                 return;
             }
             if (!rows && policy().prefill_mfma) {
-                const int tile = K::attention_masked_mfma_tile.raw(n_heads_, n_kv_heads_, head_dim_, value_dim_);
+                const int tile = K::attention_masked_mfma_tile.raw(n, n_heads_, n_kv_heads_, head_dim_, value_dim_);
                 const Tiles t = last_rows ? c.last_tiles(tile) : c.query_tiles(tile);
                 K::attention_masked_mfma(q.data, entry.keys.data, entry.values.data, tok_pos, table.dev, table.width, n_pages, window_, keep_first_, scale_,
-                                         cap_, sink, sink_dtype, t.seq, t.tok0, t.count, t.n, 0, 1, nullptr, nullptr, out.data, n_heads_, n_kv_heads_,
+                                         cap_, sink, sink_dtype, t.seq, t.tok0, t.count, t.n, tile, 0, 1, nullptr, nullptr, out.data, n_heads_, n_kv_heads_,
                                          head_dim_, value_dim_, c.stream);
                 return;
             }

@@ -300,16 +300,16 @@ int tqk_attention_masked(const void* q, const void* keys, const void* values, in
                          int n_heads, int n_kv_heads, int key_dim, int value_dim, void* stream);
 
 /* The same on the matrix cores (attention_masked_mfma.hip), bfloat16, key_dim a multiple of 8, both sizes up to 256.  n_tiles > 0:
- * tiles of up to tqk_attention_masked_mfma_tile(...) consecutive queries of one sequence (lists on the device; tok_pos and q by packed
+ * tiles of up to tile_queries = tqk_attention_masked_mfma_tile(...) consecutive queries of one sequence (lists on the device; tok_pos and q by packed
  * token, page_table by sequence of the step).  Else rows: row r is a token of its own at position tok_pos[r] whose pages are
  * page_table row r, dealt out to n_parts partitions (part_out float32 [rows, heads, n_parts, value_dim] and part_ml [rows, heads,
  * n_parts, 2] where n_parts > 1; a second kernel merges them). */
 int tqk_attention_masked_mfma_supported(int key_dim, int value_dim);
-int tqk_attention_masked_mfma_tile(int n_heads, int n_kv_heads, int key_dim, int value_dim);
+int tqk_attention_masked_mfma_tile(int n_tokens, int n_heads, int n_kv_heads, int key_dim, int value_dim);
 int tqk_attention_masked_mfma(const void* q, const void* keys, const void* values, const int32_t* tok_pos, const int32_t* page_table,
                               int table_width, int n_pages, int window, int keep_first, float scale, float cap, const void* sink,
                               int sink_dtype, const int32_t* tile_seq, const int32_t* tile_tok0, const int32_t* tile_count, int n_tiles,
-                              int n_rows, int n_parts, void* part_out, void* part_ml, void* out, int n_heads, int n_kv_heads,
+                              int tile_queries, int n_rows, int n_parts, void* part_out, void* part_ml, void* out, int n_heads, int n_kv_heads,
                               int key_dim, int value_dim, void* stream);
 
 /* out[r] = lowest index of the largest value of logits[r, :]; scratch: at least

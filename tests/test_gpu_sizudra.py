@@ -452,3 +452,20 @@ def test_a_model_of_more_windows_than_the_cache_has_groups(tmp_path_factory):
     want = S.plain_logits(cfg, w, toks)
     S.close(run_cut(eng, toks, []), want, "float32", "whole")
     S.close(run_cut(eng, toks, [70] + list(range(100, 150))), want, "float32", "a portion and single tokens")
+
+
+def test_a_step_of_many_blocks(tmp_path_factory):
+    """Sixteen prompts of 512 tokens and more in one step: enough tiles for the prompt attention's blocks of eight waves (bfloat16)."""
+    a = S.mixer(32, 8, 16, 24, 8, base=100.0, v_mix=True)
+    b = S.mixer(32, 8, 16, 24, 8, base=100.0, v_mix=True, window=100, keep_first=70, softcap=20.0)
+    cfg = S.config(80, 64, [(a, S.dense(48)), (b, S.dense(48)), (a, None)])
+    w = S.weights(cfg, seed=3, sharp=1.5)
+    eng = Engine(Model.from_dir(S.write_folder(str(tmp_path_factory.mktemp("sizudra_blocks")), cfg, w), dtype="bfloat16"), max_tokens=64 * 200, max_slots=16)
+    reqs = [S.tokens(512 + 3 * i, cfg["vocab"], 60 + i) for i in range(16)]
+    slots = [eng.open() for _ in reqs]
+    got = eng.step([(s, t, [0, 255, len(t) - 2, len(t) - 1]) for s, t in zip(slots, reqs)])
+    for i, t in enumerate(reqs):
+        want = S.plain_logits(cfg, w, t)[[0, 255, len(t) - 2, len(t) - 1]]
+        S.close(got[4 * i:4 * i + 4], want, "bfloat16", "request %d" % i, spare=0)
+    for s in slots:
+        eng.close(s)
